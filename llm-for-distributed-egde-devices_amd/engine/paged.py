@@ -16,6 +16,7 @@ Per run:
   lat  [pages, page, 1, kv_rank + R]                            latent attention: normed latent | rotated
       shared key part; a layer that reads another layer's cache holds the same tensor as that run
   canon1 / canon2 [slots, taps - 1, width] fp32                 last inputs of the sublayers' input convolutions
+  k = v [pages, page, kv heads, D]                              attention whose values are its keys: one tensor
 and, for models whose embedding looks at the previous token, ``prev_tok`` int64 [slots].
 A slot's recurrent rows are not cleared on release: a portion that starts at position 0 ignores
 what the slot held (the kernels start from zero there).
@@ -48,8 +49,12 @@ class PagedCache:
         for r, s in enumerate(run_specs):
             rc = RunCache()
             latent, delta = getattr(s, "latent", None), getattr(s, "delta", None)
-            if getattr(s, "attn", None) is None:             # a post-norm layer: one mixer of either kind
-                if latent is not None:
+            if getattr(s, "attn", None) is None:             # a layer with one mixer of either kind
+                chunk_attn = getattr(s, "chunk_attn", None)
+                if chunk_attn is not None:                   # the values are the keys: one row per token serves both
+                    rc.k = rc.v = torch.zeros(num_pages, page, chunk_attn.kv_heads, chunk_attn.dim, dtype=dtype,
+                                              device=device)
+                elif latent is not None:
                     src = s.latent.kv_from
                     if src is None:
                         rc.lat = torch.zeros(num_pages, page, 1, s.latent.cache_dim, dtype=dtype, device=device)

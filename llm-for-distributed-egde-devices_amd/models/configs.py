@@ -11,8 +11,11 @@ Families (dims are public HF configs):
   * BERT (MiniLM-L6)     — bidirectional encoder used as the sentence embedder
                            (combine_model_fp_updated.py:70-73,179)
   * layer-spec layouts   — per-layer descriptions (``layer_specs``): Nudadra (windowed attention with
-                           pooled blocks beside a Mamba-2 mixer) and Pagonex (latent attention and
-                           gated delta-rule layers with mixture-of-experts feed-forwards)
+                           pooled blocks beside a Mamba-2 mixer), Pagonex (latent attention and
+                           gated delta-rule layers with mixture-of-experts feed-forwards) and Vetevik
+                           (chunked attention with a sink and a distance bias, a gated delta rule
+                           with one decay per head, sigmoid-routed experts, norms on both sides of
+                           every sublayer)
 A single ``ModelConfig`` describes all decoder families; ``DecoderLM`` interprets the flags.
 """
 from __future__ import annotations
@@ -103,18 +106,51 @@ class LatentAttnSpec:
 
 
 @dataclass
+class ChunkAttnSpec:
+    """Grouped-query softmax attention inside chunks of ``chunk`` positions counted from the start of
+    the sequence (query i sees j <= i with floor(i / chunk) == floor(j / chunk); None: plain causal).
+    Scores (q . k) scale are capped as ``softcap`` tanh(score / softcap) (None: no cap), then lose
+    slope_h (i - j) with slope_h = 2^(-8 (h + 1) / heads) (``distance_bias``); the softmax denominator
+    also holds exp(sink_h), a learned number per head without key or value (``sink``).  The values
+    are the keys themselves (``value_is_key``: one cached row per token serves both), no rotation.
+    The concatenated heads are multiplied element by element with sigmoid(W_g h) (``gate``)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    scale: float
+    chunk: Optional[int] = None
+    softcap: Optional[float] = None
+    distance_bias: bool = True
+    sink: bool = True
+    value_is_key: bool = True
+    gate: bool = True
+
+    @property
+    def vdim(self) -> int:
+        return self.dim
+
+    @property
+    def proj_sizes(self):
+        """Row blocks of the fused input projection: q | k | gate."""
+        return (self.heads * self.dim, self.kv_heads * self.dim, self.heads * self.dim if self.gate else 0)
+
+
+@dataclass
 class DeltaSpec:
-    """Gated delta rule with one decay per head and key channel: a [dim, vdim] fp32 state per head,
-    q / k shared by ``heads / kv_heads`` heads, a causal depthwise convolution of ``conv`` taps + silu
-    over q | k | v, unit-length q and k, low-rank decay (``decay_rank``) and output-gate
-    (``gate_rank``) projections, an RMS norm per head with one weight vector shared by the heads."""
+    """Gated delta rule: a [dim, vdim] fp32 state per head, q / k shared by ``heads / kv_heads`` heads,
+    a causal depthwise convolution of ``conv`` taps + silu over q | k | v, unit-length q and k, an RMS
+    norm per head with one weight vector shared by the heads.  ``decay`` "channel": one decay per
+    head and key channel through a low-rank projection (``decay_rank``) with a sigmoid output gate
+    through another (``gate_rank``); "head": one decay per head from a plain projection
+    (exp(-exp(A_log) softplus(W_a h + dt_bias))) with a full-rank silu output gate (ranks 0)."""
     heads: int
     kv_heads: int
     dim: int
     vdim: int
     conv: int
-    decay_rank: int
-    gate_rank: int
+    decay_rank: int = 0
+    gate_rank: int = 0
+    decay: str = "channel"
 
     @property
     def conv_channels(self) -> int:
@@ -122,24 +158,33 @@ class DeltaSpec:
 
     @property
     def in_sizes(self):
-        """Row blocks of the fused input projection: q | k | v | beta | decay down | gate down."""
+        """Row blocks of the fused input projection: q | k | v | beta | decay down | gate down
+        (per-head decays: q | k | v | beta | decay | gate)."""
+        if self.decay == "head":
+            return (self.kv_heads * self.dim, self.kv_heads * self.dim, self.heads * self.vdim, self.heads,
+                    self.heads, self.heads * self.vdim)
         return (self.kv_heads * self.dim, self.kv_heads * self.dim, self.heads * self.vdim, self.heads,
                 self.decay_rank, self.gate_rank)
 
 
 @dataclass
 class MoESpec:
-    """Mixture of clamped gated-linear experts: softmax router over ``experts``, the ``top`` largest
-    renormalised and multiplied by ``scale``; an optional shared expert of width ``shared_ff`` runs
-    for every token.  Expert: g = min(W_g h, limit), u = clamp(W_u h, +-limit),
-    W_d (g sigmoid(1.702 g) (u + 1))."""
+    """Mixture of gated-linear experts.  ``router`` "softmax": softmax over ``experts``, the ``top``
+    largest renormalised and multiplied by ``scale``; "sigmoid": scores sigmoid(W_r h), the ``top``
+    largest taken as they are.  ``act`` "glu_clamp": g = min(W_g h, limit), u = clamp(W_u h, +-limit),
+    W_d (g sigmoid(1.702 g) (u + 1)); "silu_glu": W_d (silu(W_g h) (W_u h)).  ``weight_on`` "output":
+    the result is sum_k w_k expert_k(h); "input": sum_k expert_k(w_k h).  An optional shared expert of
+    width ``shared_ff`` runs for every token."""
     experts: int
     top: int
     scale: float
     ff: int
-    limit: float
+    limit: float = 0.0
     shared_ff: int = 0
     shared_limit: float = 0.0
+    router: str = "softmax"
+    act: str = "glu_clamp"
+    weight_on: str = "output"
 
 
 @dataclass
@@ -147,7 +192,8 @@ class LayerSpec:
     """One layer of a ``layer_specs`` model: the mixer kind with its branches, and the feed-forward
     (``ff``: dense width, ``moe``: mixture of experts; neither: the layer has no feed-forward)."""
     mixer: str                               # "parallel": attention and state-space side by side;
-                                             # "latent_attention" / "channel_delta": one mixer, norm on the sublayer's output
+                                             # "latent_attention" / "channel_delta": one mixer, norm on the sublayer's output;
+                                             # "chunk_attention" / "head_delta": one mixer, norms on both sides of each sublayer
     attn: Optional[WindowAttnSpec] = None
     ssd: Optional[SSDSpec] = None
     ff: Optional[int] = None
@@ -155,14 +201,18 @@ class LayerSpec:
     latent: Optional[LatentAttnSpec] = None
     delta: Optional[DeltaSpec] = None
     moe: Optional[MoESpec] = None
+    chunk_attn: Optional[ChunkAttnSpec] = None
 
 
 @dataclass
 class LoopSpec:
-    """Layers [start, stop) run ``times`` times in a row with the same weights."""
+    """Layers [start, stop) run ``times`` times in a row with the same weights.  ``entry``: what
+    happens to the stream right before each pass but the first: "project" (W_in [x ; x0] + step[t])
+    or "add_embed" (x + x0), x0 being the embedding output."""
     start: int
     stop: int
     times: int
+    entry: str = "project"
 
 
 @dataclass
@@ -203,6 +253,10 @@ class ModelConfig:
     canon_taps: int = 0
     bigram: Optional[dict] = None            # {"buckets", "mul_prev", "mul_cur"}
     logit_scale: float = 1.0
+    # arch "vetevik": norms in ``norm_groups`` parts before and after every sublayer, whose normed output
+    # is multiplied by ``residual_mult`` before it joins the stream
+    norm_groups: int = 1
+    residual_mult: float = 1.0
 
     def layer_runs(self) -> List[tuple]:
         """[(layer index, pass number or None)] in execution order; every run has its own cache."""
@@ -550,6 +604,79 @@ def to_pagonex_config(cfg: ModelConfig) -> dict:
     return out
 
 
+def from_vetevik_config(c: dict) -> ModelConfig:
+    """The Vetevik layout of ``config.json``: ``layers`` (``type`` = ``delta`` or ``attention``, ``mixer``
+    sizes and constants, ``mlp`` = mixture of experts or null), ``loop``, ``norm.eps`` / ``norm.groups``,
+    ``residual_mult``, ``vocab``, ``width``.  The embedding table is also the output projection."""
+    specs = []
+    for l in c["layers"]:
+        m, kind = l["mixer"], l["type"]
+        ca = dl = None
+        if kind == "attention":
+            mask = m.get("mask") or {}
+            if m.get("vdim") is not None and int(m["vdim"]) != int(m["dim"]):
+                raise ValueError("the values are the keys: vdim must equal dim")
+            ca = ChunkAttnSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
+                               scale=float(m["scale"]),
+                               chunk=int(mask["size"]) if mask.get("size") is not None else None,
+                               softcap=float(m["softcap"]) if m.get("softcap") else None)
+            if ca.heads % ca.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+        elif kind == "delta":
+            dl = DeltaSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
+                           vdim=int(m["vdim"]), conv=int(m["conv"]), decay="head")
+            if dl.heads % dl.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+        else:
+            raise ValueError(f"unsupported layer type {kind!r}")
+        mlp, moe = l.get("mlp") or None, None
+        if mlp:
+            if mlp.get("kind") != "moe":
+                raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}")
+            r = mlp["router"]
+            moe = MoESpec(experts=int(r["experts"]), top=int(r["top"]), scale=1.0, ff=int(mlp["expert"]["ff"]),
+                          router="sigmoid", act="silu_glu", weight_on="input")
+        specs.append(LayerSpec("chunk_attention" if ca else "head_delta", delta=dl, moe=moe, chunk_attn=ca))
+    lp = c.get("loop") or None
+    if lp and not (0 <= int(lp["start"]) < int(lp["stop"]) <= len(specs) and int(lp["times"]) >= 1):
+        raise ValueError("loop: 0 <= start < stop <= layers and times >= 1")
+    first = specs[0].chunk_attn or specs[0].delta
+    return ModelConfig(arch="vetevik", vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), num_layers=len(specs),
+                       num_heads=first.heads, num_kv_heads=first.kv_heads, intermediate_size=0, head_dim=first.dim,
+                       max_position_embeddings=1 << 20, norm="rms_group", norm_eps=float(c["norm"]["eps"]),
+                       act="silu_glu", pos_emb="none", tie_word_embeddings=True, name=c.get("name", "vetevik"),
+                       layer_specs=specs,
+                       loop=LoopSpec(int(lp["start"]), int(lp["stop"]), int(lp["times"]), "add_embed") if lp else None,
+                       norm_groups=int(c["norm"].get("groups", 1)), residual_mult=float(c.get("residual_mult", 1.0)))
+
+
+def to_vetevik_config(cfg: ModelConfig) -> dict:
+    """Inverse of ``from_vetevik_config``."""
+    layers = []
+    for s in cfg.layer_specs:
+        if s.chunk_attn is not None:
+            a = s.chunk_attn
+            m = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.dim, "scale": a.scale}
+            if a.softcap:
+                m["softcap"] = a.softcap
+            if a.chunk is not None:
+                m["mask"] = {"size": a.chunk}
+            kind = "attention"
+        else:
+            d = s.delta
+            m = {"heads": d.heads, "kv_heads": d.kv_heads, "dim": d.dim, "vdim": d.vdim, "conv": d.conv}
+            kind = "delta"
+        mlp = None
+        if s.moe is not None:
+            mlp = {"kind": "moe", "router": {"experts": s.moe.experts, "top": s.moe.top}, "expert": {"ff": s.moe.ff}}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    out = {"architecture": "Vetevik", "vocab": cfg.vocab_size, "width": cfg.hidden_size, "layers": layers,
+           "norm": {"eps": cfg.norm_eps, "groups": cfg.norm_groups}, "residual_mult": cfg.residual_mult}
+    if cfg.loop is not None:
+        out["loop"] = {"start": cfg.loop.start, "stop": cfg.loop.stop, "times": cfg.loop.times}
+    return out
+
+
 def from_hf_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
     """Map a ``config.json`` onto ModelConfig (Hugging Face ``model_type`` layouts, or an
     ``architecture`` key naming a per-layer layout; ``shapes``: the checkpoint's tensor shapes, for
@@ -558,6 +685,8 @@ def from_hf_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
         return from_nudadra_config(c)
     if str(c.get("architecture", "")).lower() == "pagonex":
         return from_pagonex_config(c, shapes)
+    if str(c.get("architecture", "")).lower() == "vetevik":
+        return from_vetevik_config(c)
     mt = c.get("model_type")
     eos = c.get("eos_token_id")
     if isinstance(eos, list):

@@ -159,11 +159,10 @@ def load_hf_model(path: str, dtype=torch.bfloat16, device=None, first: int = 0,
     cfg = from_hf_dir(path)
     if cfg.layer_specs is not None:
         # layer-spec checkpoints: names l<i>.norm1 / l<i>.mix.* / l<i>.mlp.* / head
-        from .hybrid import HybridLM, convert_nudadra_tensors, convert_pagonex_tensors, load_into_hybrid
+        from .hybrid import CONVERTERS, HybridLM, load_into_hybrid
         assert first == 0 and last in (None, cfg.num_layers), "layer-spec models load whole"
         model = HybridLM(cfg, dtype=dtype, device=device).eval()
-        convert = convert_pagonex_tensors if cfg.arch == "pagonex" else convert_nudadra_tensors
-        return load_into_hybrid(model, convert(cfg, dict(_iter_checkpoint(path))))
+        return load_into_hybrid(model, CONVERTERS[cfg.arch][0](cfg, dict(_iter_checkpoint(path))))
     model = DecoderLM(cfg, dtype=dtype, device=device, first=first, last=last).eval()
     tensors = convert_hf_tensors(cfg, _iter_checkpoint(path), first, model.last)
     return load_into(model, tensors)
@@ -251,15 +250,15 @@ def save_hf_model(model: DecoderLM, path: str, shard_bytes: int = 4 << 30) -> st
     """Write ``config.json`` + safetensors shards readable by both edgellm and transformers
     (layer-spec models: their own config layout and tensor names)."""
     from safetensors.torch import save_file
-    from .configs import to_hf_config, to_nudadra_config, to_pagonex_config
+    from .configs import to_hf_config, to_nudadra_config, to_pagonex_config, to_vetevik_config
     os.makedirs(path, exist_ok=True)
     spec_model = model.cfg.layer_specs is not None
-    to_spec = to_pagonex_config if model.cfg.arch == "pagonex" else to_nudadra_config
+    to_spec = {"pagonex": to_pagonex_config, "vetevik": to_vetevik_config}.get(model.cfg.arch, to_nudadra_config)
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(to_spec(model.cfg) if spec_model else to_hf_config(model.cfg), f, indent=2)
     if spec_model:
-        from .hybrid import export_nudadra_tensors, export_pagonex_tensors
-        tensors = export_pagonex_tensors(model) if model.cfg.arch == "pagonex" else export_nudadra_tensors(model)
+        from .hybrid import CONVERTERS
+        tensors = CONVERTERS[model.cfg.arch][1](model)
     else:
         tensors = export_hf_tensors(model)
     shards, cur, size = [], {}, 0

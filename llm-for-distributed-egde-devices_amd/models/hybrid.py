@@ -1,4 +1,4 @@
-"""Layer-spec language models (arch "nudadra", "pagonex"): every layer is described by its own
+"""Layer-spec language models (arch "nudadra", "pagonex", "vetevik"): every layer is described by its own
 entry of ``ModelConfig.layer_specs``, a span of layers may run several times in a row, and the
 residual stream is fp32.
 
@@ -7,6 +7,12 @@ x <- x + LN2(ff(x + conv2(x))): the sublayers read the stream itself plus a caus
 convolution of it over time, and the LayerNorm sits on each sublayer's output.  The mixer is latent
 attention or a gated delta rule (models/mixers.py), the feed-forward a mixture of experts
 (models/moe.py).  The embedding adds a hashed (previous token, token) row; the logits are scaled.
+
+Per layer (norms on both sides, ``SandwichLayer``):  x <- x + m N1b(mixer(N1(x))) ;
+x <- x + m N2b(ff(N2(x))), every N an RMS norm in groups with its own weight vector and m one number
+for the model.  The mixer is chunked attention with a sink or a gated delta rule with a decay per
+head, the feed-forward a sigmoid-routed mixture of experts; a looped span adds the embedding rows
+to the stream before every pass but the first; the embedding table is the output projection.
 
 Per layer (parallel form):  h = norm(x) ;  x <- x + mixer(h) + ff(h), with one norm whose gain is a
 single number, a ``ParallelMixer`` (models/mixers.py) and a squared-ReLU feed-forward.  The
@@ -31,8 +37,8 @@ import torch.nn as nn
 
 from ..ops import seqmix
 from .configs import LayerSpec, ModelConfig
-from .layers import Linear, RowLayerNorm, ScalarNorm
-from .mixers import ChannelDeltaMixer, LatentAttention, ParallelMixer
+from .layers import GroupRMSNorm, Linear, RowLayerNorm, ScalarNorm
+from .mixers import ChannelDeltaMixer, ChunkAttention, HeadDeltaMixer, LatentAttention, ParallelMixer
 from .moe import MoEFeedForward
 
 
@@ -90,9 +96,41 @@ class PostNormLayer(nn.Module):
         return x
 
 
+class SandwichLayer(nn.Module):
+    """One mixer (chunked attention or a gated delta rule with per-head decays) and an optional
+    mixture-of-experts feed-forward, each between two grouped RMS norms: the sublayer reads the normed
+    stream, and ``residual_mult`` times the norm of its output joins the fp32 stream."""
+
+    def __init__(self, cfg: ModelConfig, spec: LayerSpec, idx: int, dtype, device):
+        super().__init__()
+        W, eps, groups = cfg.hidden_size, cfg.norm_eps, cfg.norm_groups
+        self.idx, self.spec, self.dtype, self.mult = idx, spec, dtype, cfg.residual_mult
+        if spec.mixer == "chunk_attention":
+            self.mix = ChunkAttention(spec.chunk_attn, W, dtype, device)
+        elif spec.mixer == "head_delta":
+            self.mix = HeadDeltaMixer(spec.delta, W, eps, dtype, device)
+        else:
+            raise ValueError(spec.mixer)
+        N = lambda: GroupRMSNorm(W, groups, eps, device)
+        self.norm1, self.norm1b = N(), N()
+        self.ff = MoEFeedForward(spec.moe, W, dtype, device) if spec.moe is not None else None
+        if self.ff is not None:
+            self.norm2, self.norm2b = N(), N()
+
+    def forward(self, x: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        self.norm1b.add_to(x, self.mix(self.norm1(x, self.dtype), meta, run), self.mult)
+        if self.ff is not None:
+            shared, parts, wts = self.ff(self.norm2(x, self.dtype))
+            self.norm2b.add_to(x, shared, self.mult, parts, wts)
+        return x
+
+
 def _make_layer(cfg: ModelConfig, spec: LayerSpec, idx: int, dtype, device) -> nn.Module:
-    return HybridLayer(cfg, spec, idx, dtype, device) if spec.mixer == "parallel" else \
-        PostNormLayer(cfg, spec, idx, dtype, device)
+    if spec.mixer == "parallel":
+        return HybridLayer(cfg, spec, idx, dtype, device)
+    if spec.mixer in ("chunk_attention", "head_delta"):
+        return SandwichLayer(cfg, spec, idx, dtype, device)
+    return PostNormLayer(cfg, spec, idx, dtype, device)
 
 
 class HybridLM(nn.Module):
@@ -111,13 +149,16 @@ class HybridLM(nn.Module):
         if cfg.bigram:
             self.bigram = nn.Parameter(torch.empty(cfg.bigram["buckets"] + 1, W, dtype=dtype, device=device),
                                        requires_grad=False)
-        if cfg.loop is not None:
+        if cfg.loop is not None and cfg.loop.entry == "project":
             self.loop_in = Linear(2 * W, W, False, dtype, device)
             self.loop_step = nn.Parameter(torch.zeros(cfg.loop.times, W, dtype=torch.float32, device=device),
                                           requires_grad=False)
         self.final_norm = ScalarNorm(cfg.norm_eps, device) if cfg.norm == "rms_scalar" else \
+            GroupRMSNorm(W, cfg.norm_groups, cfg.norm_eps, device) if cfg.norm == "rms_group" else \
             RowLayerNorm(W, cfg.norm_eps, device)
         self.lm_head = Linear(W, cfg.vocab_size, False, dtype, device)
+        if cfg.tie_word_embeddings:                      # the embedding table is the output projection
+            self.lm_head.weight = self.embed
 
     @property
     def device(self):
@@ -151,7 +192,11 @@ class HybridLM(nn.Module):
         x = x0.clone() if cfg.loop is not None else x0
         for r, (i, t) in enumerate(self.runs):
             if t is not None and i == cfg.loop.start:
-                x = seqmix.linear_f32(seqmix.cat_cast(x, x0, self.dtype), self.loop_in.weight, self.loop_step[t])
+                if cfg.loop.entry == "add_embed":
+                    if t > 0:                            # every pass but the first starts from x + the embedding rows
+                        x.add_(x0)
+                else:
+                    x = seqmix.linear_f32(seqmix.cat_cast(x, x0, self.dtype), self.loop_in.weight, self.loop_step[t])
             x = self.layers[i](x, meta, cache.run(r))
             if taps is not None:
                 taps.append(x.clone())
@@ -314,6 +359,70 @@ def export_pagonex_tensors(model: "HybridLM") -> Dict[str, torch.Tensor]:
     return {k: v.to(torch.bfloat16).contiguous() for k, v in out.items()}
 
 
+def convert_vetevik_tensors(cfg: ModelConfig, t: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    """Checkpoint names of the Vetevik layout (``l<i>.norm1b``, ``l<i>.mix.q.conv``, ``l<i>.mlp.e<k>.gate``
+    ...) -> this package's parameter names: fused input projections, stacked expert weights."""
+    out = {"embed": t["embed"], "final_norm.weight": t["final.norm"]}
+    for i, spec in enumerate(cfg.layer_specs):
+        p, o = f"l{i}.", f"layers.{i}."
+        M, m = p + "mix.", o + "mix."
+        for n in ("1", "1b", "2", "2b") if spec.moe is not None else ("1", "1b"):
+            out[o + f"norm{n}.weight"] = t[p + f"norm{n}"]
+        if spec.chunk_attn is not None:
+            out[m + "proj_in.weight"] = torch.cat([t[M + n] for n in ("q", "k", "g")], 0)
+            out[m + "sink"] = t[M + "sink"]
+        else:
+            out[m + "proj_in.weight"] = torch.cat([t[M + n] for n in ("q", "k", "v", "b", "a", "g")], 0)
+            out[m + "conv_w"] = torch.cat([t[M + n + ".conv"] for n in ("q", "k", "v")], 0)
+            out[m + "dt_bias"], out[m + "A_log"], out[m + "norm_w"] = t[M + "dt_bias"], t[M + "A_log"], t[M + "norm"]
+        out[m + "o.weight"] = t[M + "o"]
+        if spec.moe is not None:
+            e, F_, f = spec.moe, p + "mlp.", o + "ff."
+            out[f + "router"] = t[F_ + "router"]
+            out[f + "w_gu"] = torch.stack([torch.cat([t[f"{F_}e{k}.gate"], t[f"{F_}e{k}.up"]], 0) for k in range(e.experts)])
+            out[f + "w_down"] = torch.stack([t[f"{F_}e{k}.down"] for k in range(e.experts)])
+    return out
+
+
+def export_vetevik_tensors(model: "HybridLM") -> Dict[str, torch.Tensor]:
+    """Inverse of ``convert_vetevik_tensors`` (checkpoint names, 16-bit storage)."""
+    cfg = model.cfg
+    p = {k: v.detach() for k, v in model.named_parameters()}
+    out = {"embed": p["embed"], "final.norm": p["final_norm.weight"]}
+    for i, spec in enumerate(cfg.layer_specs):
+        q, o = f"l{i}.", f"layers.{i}."
+        M, m = q + "mix.", o + "mix."
+        for n in ("1", "1b", "2", "2b") if spec.moe is not None else ("1", "1b"):
+            out[q + f"norm{n}"] = p[o + f"norm{n}.weight"]
+        w = p[m + "proj_in.weight"]
+        if spec.chunk_attn is not None:
+            a = spec.chunk_attn
+            for n, part in zip(("q", "k", "g"), torch.split(w, list(a.proj_sizes), 0)):
+                out[M + n] = part
+            out[M + "sink"] = p[m + "sink"]
+        else:
+            d = spec.delta
+            for n, part in zip(("q", "k", "v", "b", "a", "g"), torch.split(w, list(d.in_sizes), 0)):
+                out[M + n] = part
+            GN = d.kv_heads * d.dim
+            for n, part in zip(("q", "k", "v"), torch.split(p[m + "conv_w"], [GN, GN, d.heads * d.vdim], 0)):
+                out[M + n + ".conv"] = part
+            out[M + "dt_bias"], out[M + "A_log"], out[M + "norm"] = p[m + "dt_bias"], p[m + "A_log"], p[m + "norm_w"]
+        out[M + "o"] = p[m + "o.weight"]
+        if spec.moe is not None:
+            e, F_, f = spec.moe, q + "mlp.", o + "ff."
+            out[F_ + "router"] = p[f + "router"]
+            for k in range(e.experts):
+                out[f"{F_}e{k}.gate"], out[f"{F_}e{k}.up"] = p[f + "w_gu"][k, :e.ff], p[f + "w_gu"][k, e.ff:]
+                out[f"{F_}e{k}.down"] = p[f + "w_down"][k]
+    return {k: v.to(torch.bfloat16).contiguous() for k, v in out.items()}
+
+
+CONVERTERS = {"nudadra": (convert_nudadra_tensors, export_nudadra_tensors),
+              "pagonex": (convert_pagonex_tensors, export_pagonex_tensors),
+              "vetevik": (convert_vetevik_tensors, export_vetevik_tensors)}
+
+
 @torch.no_grad()
 def load_into_hybrid(model: HybridLM, tensors: Dict[str, torch.Tensor]) -> HybridLM:
     missing = []
@@ -357,6 +466,8 @@ def init_random_hybrid_(model: HybridLM, seed: int = 0) -> HybridLM:
             v = r(*p.shape) * (0.5 if name == "bigram" else 1.0)
         elif leaf in ("q_norm", "kv_norm"):
             v = 1.0 + 0.1 * r(*p.shape)
+        elif leaf == "sink":
+            v = r(*p.shape)
         elif leaf in ("canon1", "canon2"):
             v = 0.3 * r(*p.shape)
         elif leaf == "bias" and p.dim() == 1:            # LayerNorm biases

@@ -287,6 +287,25 @@ class RowLayerNorm(nn.Module):
         return ops.seqmix.layer_norm_residual(x, y, self.weight, self.bias, self.eps, parts, part_w)
 
 
+class GroupRMSNorm(nn.Module):
+    """RMS norm in ``groups`` equal consecutive parts with a weight vector, over fp32 rows (the residual
+    stream of the layer-spec models): ``forward`` gives rows of the consumer's dtype (a norm before a
+    sublayer); ``add_to`` adds ``mult`` times the normed rows of y + sum_k part_w[:, k] parts[:, k] into
+    an fp32 stream in place (a norm on a sublayer's output)."""
+
+    def __init__(self, width: int, groups: int, eps: float, device=None):
+        super().__init__()
+        assert width % groups == 0, "the width must split into equal parts"
+        self.eps, self.groups = eps, groups
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, x: torch.Tensor, out_dtype=torch.bfloat16) -> torch.Tensor:
+        return ops.seqmix.group_rms_norm(x, self.weight, self.groups, self.eps, out_dtype)
+
+    def add_to(self, x: torch.Tensor, y, mult: float = 1.0, parts=None, part_w=None) -> torch.Tensor:
+        return ops.seqmix.group_norm_residual(x, y, self.weight, self.groups, self.eps, mult, parts, part_w)
+
+
 def act_fn(x, act: str, quant: bool):
     if quant:
         q, s = ops.activation_quant(x, act)

@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 
 from ..ops import seqmix
-from .configs import SSDSpec, WindowAttnSpec
+from .configs import ChunkAttnSpec, DeltaSpec, SSDSpec, WindowAttnSpec
 from .layers import Linear
 
 
@@ -218,3 +218,60 @@ class ChannelDeltaMixer(nn.Module):
         prep = seqmix.delta_prepare(qkv, u, C, a, self.dt_bias, self.A_log, s.heads, s.kv_heads, s.dim)
         y = seqmix.delta_rule_scan(prep, qkv, run.ssm, meta, s.heads, s.kv_heads, s.dim, s.vdim)
         return self.o(seqmix.head_norm_gate(y, z, self.norm_w, s.heads, self.eps, h.dtype))
+
+
+class ChunkAttention(nn.Module):
+    """Grouped-query attention inside chunks of the sequence whose values are its keys: one cached row
+    per token and kv head serves scores and output.  Scores are tanh-capped, lose a per-head slope
+    times the distance, and share the softmax with a learned sink per head; the concatenated heads
+    are gated element by element with sigmoid(W_g h).  One fused GEMM produces q | k | gate."""
+
+    def __init__(self, spec: ChunkAttnSpec, width: int, dtype, device):
+        super().__init__()
+        self.spec = spec
+        s = spec
+        self.proj_in = Linear(width, sum(s.proj_sizes), False, dtype, device)
+        self.sink = nn.Parameter(torch.zeros(s.heads, dtype=torch.float32, device=device), requires_grad=False) \
+            if s.sink else None
+        self.register_buffer("slopes", seqmix.distance_slopes(s.heads, device) if s.distance_bias else None,
+                             persistent=False)
+        self.o = Linear(s.heads * s.dim, width, False, dtype, device)
+
+    def forward(self, h: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        s = self.spec
+        nq, nk, ng = s.proj_sizes
+        u = self.proj_in(h)
+        q = seqmix.rope_paged_write(u[:, :nq + nk], meta, None, run.k, None, s.heads, 0)
+        a = seqmix.chunk_attention(q, u[:, nq + nk:nq + nk + ng] if ng else None, run.k, meta, s.scale, s.chunk,
+                                   s.softcap, self.slopes, self.sink)
+        return self.o(a)
+
+
+class HeadDeltaMixer(nn.Module):
+    """Gated delta rule with one decay per head: convolution + silu over q | k | v, unit-length q and
+    k, beta = sigmoid(W_b h), decay exp(-exp(A_log) softplus(W_a h + dt_bias)), the recurrence over a
+    [dim, vdim] fp32 state per head, a per-head RMS norm times silu(W_g h), and the output projection.
+    One fused GEMM produces q | k | v | beta | decay | gate."""
+
+    def __init__(self, spec: DeltaSpec, width: int, eps: float, dtype, device):
+        super().__init__()
+        assert spec.decay == "head"
+        self.spec, self.eps = spec, eps
+        s = spec
+        P = lambda *shape: nn.Parameter(torch.zeros(*shape, dtype=torch.float32, device=device), requires_grad=False)
+        self.proj_in = Linear(width, sum(s.in_sizes), False, dtype, device)
+        self.conv_w = P(s.conv_channels, s.conv)
+        self.register_buffer("conv_b", torch.zeros(s.conv_channels, dtype=torch.float32, device=device),
+                             persistent=False)             # this mixer's convolutions have no bias
+        self.dt_bias, self.A_log, self.norm_w = P(s.heads), P(s.heads), P(s.vdim)
+        self.o = Linear(s.heads * s.vdim, width, False, dtype, device)
+
+    def forward(self, h: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        s = self.spec
+        H, C = s.heads, s.conv_channels
+        u = self.proj_in(h)
+        qkv = seqmix.conv_silu(u, 0, C, self.conv_w, self.conv_b, run.conv, meta)
+        prep = seqmix.delta_prepare_head(qkv, u, C, C + H, self.dt_bias, self.A_log, H, s.kv_heads, s.dim)
+        y = seqmix.delta_rule_scan(prep, qkv, run.ssm, meta, H, s.kv_heads, s.dim, s.vdim)
+        z = u[:, C + 2 * H:C + 2 * H + H * s.vdim]
+        return self.o(seqmix.head_norm_gate(y, z, self.norm_w, H, self.eps, h.dtype, act="silu"))

@@ -1,7 +1,8 @@
 """Mixture-of-experts feed-forward for layer-spec models.
 
-Router: softmax over all experts in fp32, the ``top`` largest scores renormalised and scaled
-(``ops.seqmix.moe_route``).  Experts: clamped gated-linear units, weights stacked per layer as
+Router: softmax over all experts in fp32, the ``top`` largest scores renormalised and scaled, or
+sigmoid scores taken as they are (``ops.seqmix.moe_route``).  Experts: clamped or plain silu
+gated-linear units, the router's weight on their output or on their input, weights stacked per layer as
 ``w_gu`` [E, 2 ff, W] (gate rows, then up rows) and ``w_down`` [E, W, ff]; decode-sized steps read
 only the chosen experts' rows, prompt-sized steps sort (token, choice) pairs by expert
 (``ops.seqmix.moe_experts``).  The shared expert is a dense unit of the same form.  ``forward``
@@ -31,10 +32,14 @@ class MoEFeedForward(nn.Module):
             self.shared_down = Linear(s.shared_ff, width, False, dtype, device)
 
     def forward(self, h: torch.Tensor):
-        """h [T, W] -> (shared expert's output [T, W] or None, expert outputs [T, top, W], weights fp32 [T, top])."""
+        """h [T, W] -> (shared expert's output [T, W] or None, expert outputs [T, top, W], weights fp32
+        [T, top] still to be applied to them, or None when the experts ran on weighted inputs)."""
         s = self.spec
-        idx, wts = seqmix.moe_route(h, self.router, s.top, s.scale)
-        parts = seqmix.moe_experts(h, idx, self.w_gu, self.w_down, s.limit)
+        idx, wts = seqmix.moe_route(h, self.router, s.top, s.scale, s.router)
+        on_input = s.weight_on == "input"
+        parts = seqmix.moe_experts(h, idx, self.w_gu, self.w_down, s.limit, s.act, wts if on_input else None)
+        if on_input:
+            wts = None
         shared = None
         if s.shared_ff:
             shared = self.shared_down(seqmix.glu_clamp(self.shared_gu(h), s.shared_ff, s.shared_limit))

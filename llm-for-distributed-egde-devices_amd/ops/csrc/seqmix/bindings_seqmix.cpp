@@ -21,19 +21,28 @@ int edge_sm_gated_norm(const float* y, const void* z, int z_ld, const float* w, 
 int edge_sm_rope_write(const void* proj, int ld, const int* tok_seq, const int* tok_pos, const int* seq_slot,
                        const int* ptab, int ptab_ld, const float* cs, void* q_out, void* kp, void* vp, int rows,
                        int H, int G, int D, int Dv, int rot, int page, int f32, hipStream_t st);
+int edge_sm_group_norm(const float* x, const float* w, void* y, int rows, int W, int groups, float eps, int f32,
+                       hipStream_t st);
+int edge_sm_group_norm_residual(float* x, const void* y, const void* parts, const float* pw, int K, const float* w,
+                                int rows, int W, int groups, float eps, float mult, int f32, hipStream_t st);
+int edge_sm_glu_silu(const void* u, int ld, void* y, const float* row_w, int rows, int ff, int f32, hipStream_t st);
+int edge_sm_delta_prep_head(const void* qkv, int Cq, const void* u, int ld, int b0, int a0, const float* dt_bias,
+                            const float* A_log, float* prep, int rows, int H, int G, int N, int f32, hipStream_t st);
 int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, const int* seq_slot,
                         const int* seq_start, const int* seq_len, const int* ptab, int ptab_ld, int n, int max_blocks,
                         int G, int D, int Dv, int page, int PB, int pool, int f32, hipStream_t st);
 int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
-                      int window, int pool, int f32, int nsplit, float* part, int kld, int vld, hipStream_t st);
+                      int window, int pool, int f32, int nsplit, float* part, int kld, int vld, int chunked, float cap,
+                      const float* slopes, const float* sink, int gate_elem, hipStream_t st);
 size_t edge_sm_attention_part_floats(int rows, int H, int G, int D, int Dv, int nsplit);
 int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp,
                            const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
                            const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
                            int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
-                           int pool, int kld, int vld, hipStream_t st);
+                           int pool, int kld, int vld, int chunked, float cap, const float* slopes, const float* sink,
+                           int gate_elem, hipStream_t st);
 int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
                       const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
                       const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
@@ -59,7 +68,7 @@ int edge_sm_ln_residual(float* x, const void* y, const void* parts, const float*
 int edge_sm_rms_cols(const void* u, int ld, int c0, int C, const float* w, void* y, int rows, float eps, int f32,
                      hipStream_t st);
 int edge_sm_head_norm_gate(const float* y, const void* z, int z_ld, const float* w, void* out, int rows, int H, int P,
-                           float eps, int f32, hipStream_t st);
+                           float eps, int silu, int f32, hipStream_t st);
 int edge_sm_glu_clamp(const void* u, int ld, void* y, int rows, int ff, float limit, int f32, hipStream_t st);
 int edge_sm_latent_write(const void* u, int ld, int c0, const float* w, float eps, const void* q, const void* q_lat,
                          long ql_t, long ql_h, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
@@ -69,11 +78,12 @@ int edge_sm_delta_prep(const void* qkv, int Cq, const void* u, int ld, int b0, c
                        const float* A_log, float* prep, int rows, int H, int G, int N, int f32, hipStream_t st);
 int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, float* state, const int* seq_slot,
                        const int* seq_start, const int* seq_len, const int* seq_off, float* y, int n, int H, int G, int N,
-                       int P, int f32, hipStream_t st);
+                       int P, int GD, int f32, hipStream_t st);
 int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, float* z, int* idx, float* wts,
-                      int rows, int f32, hipStream_t st);
+                      int rows, int sigm, int f32, hipStream_t st);
 int edge_sm_moe_experts(const void* h, int W, const int* idx, int top, const void* w_gu, const void* w_down, int ff,
-                        float limit, void* y, void* out, int rows, int E, int f32, hipStream_t st);
+                        float limit, int silu, const float* in_w, void* y, void* out, int rows, int E, int f32,
+                        hipStream_t st);
 }
 
 namespace {
@@ -180,17 +190,22 @@ at::Tensor sm_gated_norm(const at::Tensor& y, const at::Tensor& z, const at::Ten
 
 at::Tensor sm_rope_write(const at::Tensor& proj, const at::Tensor& tok_seq, const at::Tensor& tok_pos,
                          const at::Tensor& seq_slot, const at::Tensor& ptab, const std::optional<at::Tensor>& rope,
-                         at::Tensor& kp, at::Tensor& vp, int64_t H, int64_t rot) {
+                         at::Tensor& kp, const std::optional<at::Tensor>& vpo, int64_t H, int64_t rot) {
   const int ld = row_ld(proj, "proj");
   chk_i32(tok_seq, "tok_seq");
   chk_i32(tok_pos, "tok_pos");
   chk_i32(seq_slot, "seq_slot");
   chk_table(ptab);
-  TORCH_CHECK(is_act(proj) && kp.scalar_type() == proj.scalar_type() && vp.scalar_type() == proj.scalar_type() &&
-                  kp.is_cuda() && vp.is_cuda() && kp.is_contiguous() && vp.is_contiguous() && kp.dim() == 4 &&
-                  vp.dim() == 4, "pages: [pages, page, G, D] in proj's dtype");
-  const int64_t T = proj.size(0), page = kp.size(1), G = kp.size(2), D = kp.size(3), Dv = vp.size(3);
-  TORCH_CHECK(vp.size(0) == kp.size(0) && vp.size(1) == page && vp.size(2) == G, "k / v pages differ");
+  TORCH_CHECK(is_act(proj) && kp.scalar_type() == proj.scalar_type() && kp.is_cuda() && kp.is_contiguous() &&
+                  kp.dim() == 4, "pages: [pages, page, G, D] in proj's dtype");
+  const int64_t T = proj.size(0), page = kp.size(1), G = kp.size(2), D = kp.size(3);
+  int64_t Dv = 0;                                            // no value pages: the keys are the values
+  if (vpo) {
+    const at::Tensor& vp = *vpo;
+    TORCH_CHECK(vp.scalar_type() == proj.scalar_type() && vp.is_cuda() && vp.is_contiguous() && vp.dim() == 4 &&
+                    vp.size(0) == kp.size(0) && vp.size(1) == page && vp.size(2) == G, "k / v pages differ");
+    Dv = vp.size(3);
+  }
   TORCH_CHECK(proj.size(1) == (H + G) * D + G * Dv, "proj: [T, (H + G) D + G Dv]");
   TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T, "token metadata: [T]");
   if (rot > 0) {
@@ -201,7 +216,8 @@ at::Tensor sm_rope_write(const at::Tensor& proj, const at::Tensor& tok_seq, cons
   auto q = at::empty({T, H, D}, proj.options());
   check(edge_sm_rope_write(proj.data_ptr(), ld, tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(),
                            seq_slot.data_ptr<int>(), ptab.data_ptr<int>(), (int)ptab.stride(0),
-                           rot > 0 ? rope->data_ptr<float>() : nullptr, q.data_ptr(), kp.data_ptr(), vp.data_ptr(), (int)T,
+                           rot > 0 ? rope->data_ptr<float>() : nullptr, q.data_ptr(), kp.data_ptr(),
+                           vpo ? vpo->data_ptr() : nullptr, (int)T,
                            (int)H, (int)G, (int)D, (int)Dv, (int)rot, (int)page, f32(proj), stream()), "sm_rope_write");
   return q;
 }
@@ -234,7 +250,9 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
                         const at::Tensor& tok_seq, const at::Tensor& tok_pos, const at::Tensor& seq_slot,
                         const at::Tensor& ptab, double scale, int64_t window, int64_t pool, int64_t max_keys,
                         const std::optional<at::Tensor>& seq_start, const std::optional<at::Tensor>& seq_len,
-                        const std::optional<at::Tensor>& seq_off, int64_t n, int64_t qtiles) {
+                        const std::optional<at::Tensor>& seq_off, int64_t n, int64_t qtiles, bool chunked, double softcap,
+                        const std::optional<at::Tensor>& slopes, const std::optional<at::Tensor>& sink) {
+  // chunked: `window` is a chunk size and the gate is [T, H * Dv] (see attn_kernel)
   chk_i32(tok_seq, "tok_seq");
   chk_i32(tok_pos, "tok_pos");
   chk_i32(seq_slot, "seq_slot");
@@ -253,8 +271,23 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
   int gate_ld = 0, PB = 0;
   if (gate) {
     gate_ld = row_ld(*gate, "gate");
-    TORCH_CHECK(gate->size(0) == T && gate->size(1) == H && gate->scalar_type() == q.scalar_type(), "gate: [T, H]");
+    TORCH_CHECK(gate->size(0) == T && gate->size(1) == (chunked ? H * Dv : H) && gate->scalar_type() == q.scalar_type(),
+                "gate: [T, H] (one per head) or [T, H Dv] (one per coordinate)");
   }
+  const float* slopes_p = nullptr;
+  const float* sink_p = nullptr;
+  if (slopes) {
+    chk_f32(*slopes, "slopes");
+    TORCH_CHECK(slopes->numel() == H, "slopes: fp32 [H]");
+    slopes_p = slopes->data_ptr<float>();
+  }
+  if (sink) {
+    chk_f32(*sink, "sink");
+    TORCH_CHECK(sink->numel() == H, "sink: fp32 [H]");
+    sink_p = sink->data_ptr<float>();
+  }
+  TORCH_CHECK(!chunked || pool == 0, "chunked attention has no pooled blocks");
+  const int gate_elem = chunked && gate ? 1 : 0;
   if (pool > 0 && window > 0) {
     TORCH_CHECK(kb && vb, "pooled entries missing");
     chk_f32(*kb, "k_pool");
@@ -279,7 +312,8 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
                                           seq_start->data_ptr<int>(), seq_len->data_ptr<int>(), seq_off->data_ptr<int>(),
                                           ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)n, (int)qtiles,
                                           (int)H, (int)G, (int)D, (int)Dv, (int)page, PB, (float)scale, (int)window,
-                                          PB ? (int)pool : 0, (int)kld, (int)vld, stream());
+                                          PB ? (int)pool : 0, (int)kld, (int)vld, chunked ? 1 : 0, (float)softcap, slopes_p,
+                                          sink_p, gate_elem, stream());
     if (rc != 1) {
       check(rc, "sm_attention_mfma");
       return out;
@@ -301,7 +335,8 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
                           tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),
                           ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)T, (int)H, (int)G, (int)D, (int)Dv,
                           (int)page, PB, (float)scale, (int)window, PB ? (int)pool : 0, f32(q), nsplit,
-                          nsplit > 1 ? part.data_ptr<float>() : nullptr, (int)kld, (int)vld, stream()), "sm_attention");
+                          nsplit > 1 ? part.data_ptr<float>() : nullptr, (int)kld, (int)vld, chunked ? 1 : 0, (float)softcap,
+                          slopes_p, sink_p, gate_elem, stream()), "sm_attention");
   return out;
 }
 
@@ -473,7 +508,7 @@ at::Tensor sm_rms_cols(const at::Tensor& u, int64_t c0, int64_t C, const at::Ten
 }
 
 at::Tensor sm_head_norm_gate(const at::Tensor& y, const at::Tensor& z, const at::Tensor& w, int64_t heads, double eps,
-                             bool out_f32) {
+                             bool out_f32, bool silu) {
   chk_f32(y, "y");
   chk_f32(w, "weight");
   const int z_ld = row_ld(z, "z");
@@ -483,7 +518,8 @@ at::Tensor sm_head_norm_gate(const at::Tensor& y, const at::Tensor& z, const at:
   c10::hip::HIPGuardMasqueradingAsCUDA guard(y.device());
   auto out = at::empty({y.size(0), y.size(1)}, z.options());
   check(edge_sm_head_norm_gate(y.data_ptr<float>(), z.data_ptr(), z_ld, w.data_ptr<float>(), out.data_ptr(), (int)y.size(0),
-                               (int)heads, (int)(y.size(1) / heads), (float)eps, f32(z), stream()), "sm_head_norm_gate");
+                               (int)heads, (int)(y.size(1) / heads), (float)eps, silu ? 1 : 0, f32(z), stream()),
+        "sm_head_norm_gate");
   return out;
 }
 
@@ -565,8 +601,11 @@ at::Tensor sm_delta_scan(const at::Tensor& prep, const at::Tensor& qkv, at::Tens
   chk_act2(qkv, "qkv");
   for (const at::Tensor* t : {&seq_slot, &seq_start, &seq_len, &seq_off}) chk_i32(*t, "metadata");
   const int64_t T = qkv.size(0);
-  TORCH_CHECK(prep.dim() == 2 && prep.size(0) == T && prep.size(1) == 2 * G * N + H * N + H &&
+  // a decay per head and key channel (H N numbers a row) or one per head (H numbers)
+  TORCH_CHECK(prep.dim() == 2 && prep.size(0) == T &&
+                  (prep.size(1) == 2 * G * N + H * N + H || prep.size(1) == 2 * G * N + 2 * H) &&
                   qkv.size(1) == 2 * G * N + H * P, "prep [T, q | k | decay | beta], qkv [T, q | k | v]");
+  const int GD = prep.size(1) == 2 * G * N + H * N + H ? (int)N : 1;
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == N && state.size(3) == P,
               "state: fp32 [slots, heads, N, P]");
   TORCH_CHECK(seq_slot.numel() >= n && seq_start.numel() >= n && seq_len.numel() >= n && seq_off.numel() >= n,
@@ -575,12 +614,13 @@ at::Tensor sm_delta_scan(const at::Tensor& prep, const at::Tensor& qkv, at::Tens
   auto y = at::empty({T, H * P}, prep.options());
   check(edge_sm_delta_scan(prep.data_ptr<float>(), (int)prep.size(1), qkv.data_ptr(), (int)qkv.size(1), state.data_ptr<float>(),
                            seq_slot.data_ptr<int>(), seq_start.data_ptr<int>(), seq_len.data_ptr<int>(),
-                           seq_off.data_ptr<int>(), y.data_ptr<float>(), (int)n, (int)H, (int)G, (int)N, (int)P, f32(qkv),
-                           stream()), "sm_delta_scan");
+                           seq_off.data_ptr<int>(), y.data_ptr<float>(), (int)n, (int)H, (int)G, (int)N, (int)P, GD,
+                           f32(qkv), stream()), "sm_delta_scan");
   return y;
 }
 
-std::tuple<at::Tensor, at::Tensor> sm_moe_route(const at::Tensor& h, const at::Tensor& router, int64_t top, double scale) {
+std::tuple<at::Tensor, at::Tensor> sm_moe_route(const at::Tensor& h, const at::Tensor& router, int64_t top, double scale,
+                                                bool sigm) {
   chk_act2(h, "h");
   chk_f32(router, "router");
   TORCH_CHECK(router.dim() == 2 && router.size(1) == h.size(1), "router: fp32 [E, W]");
@@ -589,13 +629,13 @@ std::tuple<at::Tensor, at::Tensor> sm_moe_route(const at::Tensor& h, const at::T
   auto wts = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
   auto z = at::empty({h.size(0), router.size(0)}, wts.options());
   check(edge_sm_moe_route(h.data_ptr(), (int)h.size(1), router.data_ptr<float>(), (int)router.size(0), (int)top, (float)scale,
-                          z.data_ptr<float>(), idx.data_ptr<int>(), wts.data_ptr<float>(), (int)h.size(0), f32(h), stream()),
-        "sm_moe_route");
+                          z.data_ptr<float>(), idx.data_ptr<int>(), wts.data_ptr<float>(), (int)h.size(0), sigm ? 1 : 0,
+                          f32(h), stream()), "sm_moe_route");
   return {idx, wts};
 }
 
 at::Tensor sm_moe_experts(const at::Tensor& h, const at::Tensor& idx, const at::Tensor& w_gu, const at::Tensor& w_down,
-                          double limit) {
+                          double limit, bool silu, const std::optional<at::Tensor>& in_w) {
   chk_act2(h, "h");
   chk_i32(idx, "idx");
   const int64_t T = h.size(0), W = h.size(1);
@@ -605,13 +645,94 @@ at::Tensor sm_moe_experts(const at::Tensor& h, const at::Tensor& idx, const at::
                   w_down.size(1) == W && w_down.size(2) == w_gu.size(1) / 2 && w_gu.scalar_type() == h.scalar_type() &&
                   w_down.scalar_type() == h.scalar_type(), "experts: w_gu [E, 2 ff, W], w_down [E, W, ff]");
   const int64_t top = idx.size(1), ff = w_gu.size(1) / 2;
+  if (in_w) {
+    chk_f32(*in_w, "in_w");
+    TORCH_CHECK(silu && in_w->numel() == T * top, "in_w: fp32 [T, top], with the silu unit only");
+  }
   c10::hip::HIPGuardMasqueradingAsCUDA guard(h.device());
   auto y = at::empty({T * top, ff}, h.options());
   auto out = at::empty({T, top, W}, h.options());
   check(edge_sm_moe_experts(h.data_ptr(), (int)W, idx.data_ptr<int>(), (int)top, w_gu.data_ptr(), w_down.data_ptr(), (int)ff,
-                            (float)limit, y.data_ptr(), out.data_ptr(), (int)T, (int)w_gu.size(0), f32(h), stream()),
+                            (float)limit, silu ? 1 : 0, in_w ? in_w->data_ptr<float>() : nullptr, y.data_ptr(),
+                            out.data_ptr(), (int)T, (int)w_gu.size(0), f32(h), stream()),
         "sm_moe_experts");
   return out;
+}
+
+at::Tensor sm_group_norm(const at::Tensor& x, const at::Tensor& w, int64_t groups, double eps, bool out_f32) {
+  chk_f32(x, "x");
+  chk_f32(w, "weight");
+  TORCH_CHECK(x.dim() == 2 && w.numel() == x.size(1) && groups > 0 && x.size(1) % groups == 0,
+              "x fp32 [T, W], weight [W], W a multiple of groups");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  auto y = at::empty({x.size(0), x.size(1)}, x.options().dtype(act_type(out_f32)));
+  check(edge_sm_group_norm(x.data_ptr<float>(), w.data_ptr<float>(), y.data_ptr(), (int)x.size(0), (int)x.size(1),
+                           (int)groups, (float)eps, out_f32, stream()), "sm_group_norm");
+  return y;
+}
+
+void sm_group_norm_residual(at::Tensor& x, const std::optional<at::Tensor>& y, const at::Tensor& w, int64_t groups,
+                            double eps, double mult, const std::optional<at::Tensor>& parts,
+                            const std::optional<at::Tensor>& part_w) {
+  chk_f32(x, "x");
+  chk_f32(w, "weight");
+  TORCH_CHECK(x.dim() == 2 && w.numel() == x.size(1) && groups > 0 && x.size(1) % groups == 0 && (y || parts),
+              "x fp32 [T, W], weight [W], W a multiple of groups, y or parts");
+  const int64_t T = x.size(0), W = x.size(1);
+  int is_f32 = 0, K = 0;
+  if (y) {
+    chk_act2(*y, "y");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == W, "y: [T, W]");
+    is_f32 = f32(*y);
+  }
+  if (parts) {
+    TORCH_CHECK(parts->is_cuda() && parts->is_contiguous() && is_act(*parts) && parts->dim() == 3 && parts->size(0) == T &&
+                    parts->size(2) == W && (!y || parts->scalar_type() == y->scalar_type()), "parts: [T, K, W]");
+    K = (int)parts->size(1);
+    is_f32 = f32(*parts);
+    if (part_w) {
+      chk_f32(*part_w, "part_w");
+      TORCH_CHECK(part_w->numel() == T * K, "part_w: fp32 [T, K]");
+    }
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  check(edge_sm_group_norm_residual(x.data_ptr<float>(), y ? y->data_ptr() : nullptr, parts ? parts->data_ptr() : nullptr,
+                                    parts && part_w ? part_w->data_ptr<float>() : nullptr, K, w.data_ptr<float>(), (int)T,
+                                    (int)W, (int)groups, (float)eps, (float)mult, is_f32, stream()),
+        "sm_group_norm_residual");
+}
+
+at::Tensor sm_glu_silu(const at::Tensor& u, int64_t ff, const std::optional<at::Tensor>& row_w) {
+  TORCH_CHECK(is_act(u), "u: fp32 / bf16");
+  const int ld = row_ld(u, "u");
+  TORCH_CHECK(ff >= 0 && 2 * ff <= u.size(1), "u: [T, gate | up]");
+  if (row_w) {
+    chk_f32(*row_w, "row_w");
+    TORCH_CHECK(row_w->numel() == u.size(0), "row_w: fp32 [T]");
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(u.device());
+  auto y = at::empty({u.size(0), ff}, u.options());
+  check(edge_sm_glu_silu(u.data_ptr(), ld, y.data_ptr(), row_w ? row_w->data_ptr<float>() : nullptr, (int)u.size(0),
+                         (int)ff, f32(u), stream()), "sm_glu_silu");
+  return y;
+}
+
+at::Tensor sm_delta_prep_head(const at::Tensor& qkv, const at::Tensor& u, int64_t b0, int64_t a0, const at::Tensor& dt_bias,
+                              const at::Tensor& A_log, int64_t H, int64_t G, int64_t N) {
+  chk_act2(qkv, "qkv");
+  const int ld = row_ld(u, "u");
+  chk_f32(dt_bias, "dt_bias");
+  chk_f32(A_log, "A_log");
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(u.scalar_type() == qkv.scalar_type() && u.size(0) == T && b0 >= 0 && b0 + H <= u.size(1) && a0 >= 0 &&
+                  a0 + H <= u.size(1) && qkv.size(1) >= 2 * G * N && dt_bias.numel() == H && A_log.numel() == H &&
+                  G > 0 && H % G == 0, "delta prep shapes");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(qkv.device());
+  auto prep = at::empty({T, 2 * G * N + 2 * H}, qkv.options().dtype(at::kFloat));
+  check(edge_sm_delta_prep_head(qkv.data_ptr(), (int)qkv.size(1), u.data_ptr(), ld, (int)b0, (int)a0,
+                                dt_bias.data_ptr<float>(), A_log.data_ptr<float>(), prep.data_ptr<float>(), (int)T, (int)H,
+                                (int)G, (int)N, f32(qkv), stream()), "sm_delta_prep_head");
+  return prep;
 }
 
 }  // namespace
@@ -640,4 +761,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("sm_delta_scan", &sm_delta_scan);
   m.def("sm_moe_route", &sm_moe_route);
   m.def("sm_moe_experts", &sm_moe_experts);
+  m.def("sm_group_norm", &sm_group_norm);
+  m.def("sm_group_norm_residual", &sm_group_norm_residual);
+  m.def("sm_glu_silu", &sm_glu_silu);
+  m.def("sm_delta_prep_head", &sm_delta_prep_head);
 }

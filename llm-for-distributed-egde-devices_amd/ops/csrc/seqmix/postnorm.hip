@@ -170,18 +170,20 @@ __global__ void __launch_bounds__(NT) rms_cols_kernel(const T* __restrict__ u, i
   for (int c = threadIdx.x; c < C; c += NT) stf<T>(y + (size_t)blockIdx.x * C + c, ldf<T>(ur + c) * r * w[c]);
 }
 
-// per head: y / rms(y) * w (one weight vector for all heads) * sigmoid(z)
+// per head: y / rms(y) * w (one weight vector for all heads) * sigmoid(z)  (silu: * z sigmoid(z))
 template <typename T>
 __global__ void __launch_bounds__(64) head_norm_gate_kernel(const float* __restrict__ y, const T* __restrict__ z, int z_ld,
                                                             const float* __restrict__ w, T* __restrict__ out, int H, int P,
-                                                            float eps) {
+                                                            float eps, int silu) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* yr = y + ((size_t)t * H + h) * P;
   float ss = 0.f;
   for (int c = lane; c < P; c += 64) ss += yr[c] * yr[c];
   const float r = 1.f / sqrtf(wave_sum(ss) / (float)P + eps);
-  for (int c = lane; c < P; c += 64)
-    stf<T>(out + ((size_t)t * H + h) * P + c, yr[c] * r * w[c] * sigmoidf_(ldf<T>(z + (size_t)t * z_ld + h * P + c)));
+  for (int c = lane; c < P; c += 64) {
+    const float zv = ldf<T>(z + (size_t)t * z_ld + h * P + c);
+    stf<T>(out + ((size_t)t * H + h) * P + c, yr[c] * r * w[c] * (silu ? siluf_(zv) : sigmoidf_(zv)));
+  }
 }
 
 // g sigmoid(1.702 g) (up + 1), g = min(gate, limit), up clamped to +-limit; u row = gate [ff] | up [ff]
@@ -274,6 +276,7 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// GD = decay numbers per head in a prep row: N (one per key channel) or 1 (one for the head's whole state).
 // One workgroup per (sequence, head, 16 value columns): wave w owns columns 4 w .. 4 w + 3; the 16 lanes of
 // a DPP row share one column, lane rg of the row keeping state rows rg * NR .. rg * NR + NR - 1 in
 // registers (NR = ceil(N / 16) rounded up to 4), so the two sums over rows per token (S^T k and S^T q) are
@@ -285,7 +288,7 @@ __global__ void __launch_bounds__(NT) delta_scan_kernel(const float* __restrict_
                                                         int Cq, float* __restrict__ state, const int* __restrict__ seq_slot,
                                                         const int* __restrict__ seq_start, const int* __restrict__ seq_len,
                                                         const int* __restrict__ seq_off, float* __restrict__ y, int H, int G,
-                                                        int N, int P) {
+                                                        int N, int P, int GD) {
   constexpr int NP = 16 * NR, TC = NR >= 16 ? 4 : (NR >= 8 ? 8 : 16), EL = TC * 3 * NP / NT;   // EL = 12
   constexpr int CW = 16;                                     // value columns per workgroup
   __shared__ __attribute__((aligned(16))) float rows_s[2][TC][3][NP];   // q | k | decay
@@ -293,7 +296,7 @@ __global__ void __launch_bounds__(NT) delta_scan_kernel(const float* __restrict_
   const int s = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * CW, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6, rg = lane & 15, col = wave * 4 + (lane >> 4), p = p0 + col;
   const int start = seq_start[s], len = seq_len[s], off = seq_off[s];
-  const int g = h / (H / G), GN = G * N, HN = H * N;
+  const int g = h / (H / G), GN = G * N, HN = H * GD;
   float* st = state + ((size_t)seq_slot[s] * H + h) * N * P;
   float S[NR];
 #pragma unroll
@@ -310,7 +313,7 @@ __global__ void __launch_bounds__(NT) delta_scan_kernel(const float* __restrict_
       float v = which == 2 ? 1.f : 0.f;                      // rows past N: no decay, no key, no query
       if (tt < tc && n < N) {
         const float* pr = prep + (size_t)(off + t0 + tt) * prep_ld;
-        v = which == 0 ? pr[g * N + n] : (which == 1 ? pr[GN + g * N + n] : pr[2 * GN + h * N + n]);
+        v = which == 0 ? pr[g * N + n] : (which == 1 ? pr[GN + g * N + n] : pr[2 * GN + h * GD + (GD == 1 ? 0 : n)]);
       }
       pre[i] = v;
     }
@@ -402,19 +405,24 @@ __global__ void __launch_bounds__(NT) moe_logits_kernel(const T* __restrict__ h,
 }
 
 // One wave per token: softmax over the experts' scores, then the `top` largest (lowest index on a tie),
-// divided by their sum (+ 1e-20) and multiplied by scale.
+// divided by their sum (+ 1e-20) and multiplied by scale.  sigm: the scores are sigmoid(z) and the `top`
+// largest keep their own value (times scale).
 __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ z, int E, int top, float scale,
-                                                      int* __restrict__ idx, float* __restrict__ wts) {
+                                                      int* __restrict__ idx, float* __restrict__ wts, int sigm) {
   extern __shared__ __attribute__((aligned(16))) float z_s[];   // [E]
   const size_t t = blockIdx.x;
   const int lane = threadIdx.x;
   float mx = -INFINITY;
   for (int e = lane; e < E; e += 64) { z_s[e] = z[t * E + e]; mx = fmaxf(mx, z_s[e]); }
   mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += 64) sum += expf(z_s[e] - mx);
-  sum = wave_sum(sum);
-  for (int e = lane; e < E; e += 64) z_s[e] = expf(z_s[e] - mx) / sum;
+  if (sigm) {
+    for (int e = lane; e < E; e += 64) z_s[e] = sigmoidf_(z_s[e]);
+  } else {
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) sum += expf(z_s[e] - mx);
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) z_s[e] = expf(z_s[e] - mx) / sum;
+  }
   float tot = 0.f, my_w = 0.f;
   int my_i = 0;                                              // lane k keeps the k-th choice
   for (int k = 0; k < top; ++k) {
@@ -438,16 +446,17 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
   }
   if (lane < top) {
     idx[t * top + lane] = my_i;
-    wts[t * top + lane] = my_w / (tot + 1e-20f) * scale;
+    wts[t * top + lane] = sigm ? my_w * scale : my_w / (tot + 1e-20f) * scale;
   }
 }
 
 // decode-sized steps: out row r of pair (token, choice) = act(gate_r . h, up_r . h); one wave per row at a time,
-// lanes stride the width with 8-element loads, the token's row sits in LDS as fp32
+// lanes stride the width with 8-element loads, the token's row sits in LDS as fp32.  silu: the activation is
+// silu(w gate) (w up) with w = in_w[pair] (null: 1), the unit of an input scaled by the router's weight.
 template <typename T>
 __global__ void __launch_bounds__(NT) moe_gate_up_kernel(const T* __restrict__ h, int W, const int* __restrict__ idx, int top,
                                                          const T* __restrict__ w_gu, int ff, float limit, T* __restrict__ y,
-                                                         int rows_per_wg, int E) {
+                                                         int rows_per_wg, int E, int silu, const float* __restrict__ in_w) {
   extern __shared__ __attribute__((aligned(16))) float h_s[];   // [W]
   const size_t pair = blockIdx.x, t = pair / top;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -473,7 +482,10 @@ __global__ void __launch_bounds__(NT) moe_gate_up_kernel(const T* __restrict__ h
     }
     ag = wave_sum(ag);
     au = wave_sum(au);
-    if (lane == 0) stf<T>(y + pair * ff + r, glu_clamp_f(ag, au, limit));
+    if (lane == 0) {
+      const float rw = in_w ? in_w[pair] : 1.f;
+      stf<T>(y + pair * ff + r, silu ? siluf_(rw * ag) * (rw * au) : glu_clamp_f(ag, au, limit));
+    }
   }
 }
 
@@ -572,10 +584,10 @@ int edge_sm_rms_cols(const void* u, int ld, int c0, int C, const float* w, void*
 }
 
 int edge_sm_head_norm_gate(const float* y, const void* z, int z_ld, const float* w, void* out, int rows, int H, int P,
-                           float eps, int f32, hipStream_t st) {
+                           float eps, int silu, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   SM_T(f32, hipLaunchKernelGGL(head_norm_gate_kernel<T>, dim3(rows, H), dim3(64), 0, st, y, (const T*)z, z_ld, w, (T*)out, H,
-                               P, eps));
+                               P, eps, silu));
   return (int)hipGetLastError();
 }
 
@@ -609,13 +621,13 @@ int edge_sm_delta_prep(const void* qkv, int Cq, const void* u, int ld, int b0, c
 
 int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, float* state, const int* seq_slot,
                        const int* seq_start, const int* seq_len, const int* seq_off, float* y, int n, int H, int G, int N,
-                       int P, int f32, hipStream_t st) {
+                       int P, int GD, int f32, hipStream_t st) {
   if (n == 0) return 0;
-  if (G <= 0 || H % G || N > 256) return -2;
+  if (G <= 0 || H % G || N > 256 || (GD != N && GD != 1)) return -2;
   const dim3 grid(n, H, (P + 15) / 16);
 #define SM_DS(NR)                                                                                                  \
   SM_T(f32, hipLaunchKernelGGL((delta_scan_kernel<T, NR>), grid, dim3(NT), 0, st, prep, prep_ld, (const T*)qkv, Cq, \
-                               state, seq_slot, seq_start, seq_len, seq_off, y, H, G, N, P))
+                               state, seq_slot, seq_start, seq_len, seq_off, y, H, G, N, P, GD))
   if (N <= 64) SM_DS(4);
   else if (N <= 128) SM_DS(8);
   else SM_DS(16);
@@ -625,23 +637,24 @@ int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, 
 
 // z: fp32 scratch [rows, E] (the experts' scores)
 int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, float* z, int* idx, float* wts,
-                      int rows, int f32, hipStream_t st) {
+                      int rows, int sigm, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   if (top < 1 || top > E || top > 64 || E > 8192) return -2;
   SM_T(f32, hipLaunchKernelGGL(moe_logits_kernel<T>, dim3(rows, (E + NT / 64 - 1) / (NT / 64)), dim3(NT), 0, st, (const T*)h,
                                W, router, E, z));
-  hipLaunchKernelGGL(moe_topk_kernel, dim3(rows), dim3(64), (size_t)E * 4, st, (const float*)z, E, top, scale, idx, wts);
+  hipLaunchKernelGGL(moe_topk_kernel, dim3(rows), dim3(64), (size_t)E * 4, st, (const float*)z, E, top, scale, idx, wts, sigm);
   return (int)hipGetLastError();
 }
 
 // y: scratch [rows * top, ff]; out [rows * top, W]
 int edge_sm_moe_experts(const void* h, int W, const int* idx, int top, const void* w_gu, const void* w_down, int ff,
-                        float limit, void* y, void* out, int rows, int E, int f32, hipStream_t st) {
+                        float limit, int silu, const float* in_w, void* y, void* out, int rows, int E, int f32,
+                        hipStream_t st) {
   if (rows == 0) return 0;
   if ((size_t)W * 4 > 60 * 1024 || (size_t)ff * 4 > 60 * 1024) return -3;
   const int rpw = 16;
   SM_T(f32, hipLaunchKernelGGL(moe_gate_up_kernel<T>, dim3(rows * top, (ff + rpw - 1) / rpw), dim3(NT), (size_t)W * 4, st,
-                               (const T*)h, W, idx, top, (const T*)w_gu, ff, limit, (T*)y, rpw, E));
+                               (const T*)h, W, idx, top, (const T*)w_gu, ff, limit, (T*)y, rpw, E, silu, in_w));
   SM_T(f32, hipLaunchKernelGGL(moe_down_kernel<T>, dim3(rows * top, (W + rpw - 1) / rpw), dim3(NT), (size_t)ff * 4, st,
                                (const T*)y, ff, idx, (const T*)w_down, W, (T*)out, rpw, E));
   return (int)hipGetLastError();

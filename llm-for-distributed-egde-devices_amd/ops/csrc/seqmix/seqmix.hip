@@ -141,6 +141,7 @@ __global__ void __launch_bounds__(NT) rope_write_kernel(const T* __restrict__ pr
       if (hh < H) store8<T>(q_out + (size_t)t * H * D + e, v);
       else store8<T>(kp + (prow * G + (hh - H)) * D + d, v);
     }
+    if (!vp) return;                                         // the values are the keys: nothing more to cache
     for (int e = threadIdx.x * 8; e < G * Dv; e += NT * 8)
       *reinterpret_cast<uint4*>(vp + prow * G * Dv + e) = *reinterpret_cast<const uint4*>(row + nqk + e);
     if constexpr (sizeof(T) == 4)                            // fp32 rows: the second 16 bytes of each chunk
@@ -160,6 +161,7 @@ __global__ void __launch_bounds__(NT) rope_write_kernel(const T* __restrict__ pr
     if (hh < H) stf<T>(q_out + (size_t)t * H * D + e, v);
     else stf<T>(kp + (prow * G + (hh - H)) * D + d, v);
   }
+  if (!vp) return;
   for (int e = threadIdx.x; e < G * Dv; e += NT) vp[prow * G * Dv + e] = row[nqk + e];
 }
 
@@ -197,13 +199,15 @@ __global__ void __launch_bounds__(NT) pool_kernel(const T* __restrict__ kp, cons
 // broadcast reads), (B) wave w keeps the running max / sum of heads w, w + 4, .. and turns the
 // chunk's scores into weights, (C) wave w accumulates weight x value over its quarter of the
 // chunk with lane = value coordinate (coalesced row reads).  Tokens of the window first, then the
-// pooled blocks (fp32 rows): one softmax over both.
+// pooled blocks (fp32 rows): one softmax over both.  A score may be capped (cap tanh(s / cap), cap > 0) and
+// lose slope[head] * dist, dist = the query's distance to this thread's key.
 constexpr int KC = 256;
 
 template <typename KT, int RMAX, int DVL, bool VEC>
 __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const KT* __restrict__ vbase, int cnt, int g,
                                            int kld, int vld, int D, int Dv, int R, const float* q_s, float* s_s, int* row_s,
-                                           float* m_s, float* l_s, float* a_s, int rowidx, float (&acc)[RMAX][VEC ? 8 : DVL]) {
+                                           float* m_s, float* l_s, float* a_s, int rowidx, float (&acc)[RMAX][VEC ? 8 : DVL],
+                                           float cap = 0.f, const float* sl_s = nullptr, int dist = 0) {
   constexpr int AW = VEC ? 8 : DVL;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // (A) scores
@@ -229,6 +233,14 @@ __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const K
           for (int r = 0; r < RMAX; ++r) a[r] += q_s[r * D + d] * kv;
         }
       }
+    }
+    if (cap > 0.f) {
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) a[r] = cap * tanhf(a[r] / cap);
+    }
+    if (sl_s) {
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) a[r] -= sl_s[r] * (float)dist;
     }
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) s_s[r * KC + tid] = tid < cnt ? a[r] : -INFINITY;
@@ -330,7 +342,12 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
                                                   const int* __restrict__ seq_slot, const int* __restrict__ ptab,
                                                   int ptab_ld, T* __restrict__ out, int H, int G, int D, int Dv,
                                                   int page, int PB, float scale, int window, int pool, int nsp, int nsplit,
-                                                  float* __restrict__ part, int kld, int vld) {
+                                                  float* __restrict__ part, int kld, int vld, int chunked, float cap,
+                                                  const float* __restrict__ slopes, const float* __restrict__ sink,
+                                                  int gate_elem) {
+  // chunked: `window` is a chunk size (query i sees floor(i / window) * window .. i); cap / slopes: see attn_chunk;
+  // sink: a number per query head that joins the softmax denominator (it enters as the first key split's
+  // starting maximum with sum 1 and no value); gate_elem: the gate is [T, H * Dv], one per output coordinate
   // kld / vld: elements between consecutive cached rows of kp / vp (G * D and G * Dv for separate key
   // and value pages; a latent cache whose value is a slice of the key row passes the same stride twice)
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -344,7 +361,8 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
   float* m_s = red + RMAX * Dv;              // [RMAX] x 3
   float* l_s = m_s + RMAX;
   float* a_s = l_s + RMAX;
-  int* row_s = reinterpret_cast<int*>(a_s + RMAX);   // [KC]
+  float* sl_s = a_s + RMAX;                  // [RMAX] slopes of this workgroup's heads
+  int* row_s = reinterpret_cast<int*>(sl_s + RMAX);  // [KC]
   const int i = tok_pos[t];
   const int* pt = ptab + (size_t)seq_slot[tok_seq[t]] * ptab_ld;
   for (int e = tid; e < RMAX * D; e += NT) {
@@ -352,7 +370,13 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
     q_s[e] = r < R ? ldf<T>(q + ((size_t)t * H + hq0 + r) * D + d) * scale : 0.f;
   }
   for (int e = tid; e < RMAX * Dv; e += NT) red[e] = 0.f;
-  if (tid < RMAX) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; }
+  if (tid < RMAX) {
+    const bool sk = sink && blockIdx.z == 0 && tid < R;
+    m_s[tid] = sk ? sink[hq0 + tid] : -INFINITY;
+    l_s[tid] = sk ? 1.f : 0.f;
+    a_s[tid] = 1.f;
+    sl_s[tid] = (slopes && tid < R) ? slopes[hq0 + tid] : 0.f;
+  }
   constexpr int AW = VEC ? 8 : DVL;
   float acc[RMAX][AW];
 #pragma unroll
@@ -360,9 +384,9 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
 #pragma unroll
     for (int dl = 0; dl < AW; ++dl) acc[r][dl] = 0.f;
   __syncthreads();
-  const int jlo = window > 0 ? max(0, i - window + 1) : 0;
+  const int jlo = window > 0 ? (chunked ? (i / window) * window : max(0, i - window + 1)) : 0;
   const int nt = i - jlo + 1;
-  const int nb = (window > 0 && pool > 0 && i - window + 1 > 0) ? (i - window + 1) / pool : 0;
+  const int nb = (!chunked && window > 0 && pool > 0 && i - window + 1 > 0) ? (i - window + 1) / pool : 0;
   // key chunks [ci0, ci1) of this query belong to this workgroup (blockIdx.z of nsplit; 1: all of them)
   const int nchunks = (nt + KC - 1) / KC + (nb + KC - 1) / KC, cps = (nchunks + nsplit - 1) / nsplit;
   const int ci0 = blockIdx.z * cps, ci1 = min(nchunks, ci0 + cps);
@@ -371,7 +395,8 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
     if (ci < ci0 || ci >= ci1) continue;
     const int j = jlo + c0 + tid;
     const int rowidx = c0 + tid < nt ? pt[j / page] * page + j % page : 0;
-    attn_chunk<T, RMAX, DVL, VEC>(kp, vp, min(KC, nt - c0), g, kld, vld, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
+    attn_chunk<T, RMAX, DVL, VEC>(kp, vp, min(KC, nt - c0), g, kld, vld, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc,
+                                  cap, slopes ? sl_s : nullptr, i - j);
   }
   for (int c0 = 0; c0 < nb; c0 += KC, ++ci) {
     if (ci < ci0 || ci >= ci1) continue;
@@ -419,7 +444,7 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
   for (int e = tid; e < R * Dv; e += NT) {
     const int r = e / Dv, h = hq0 + r;
     float o = red[e] / l_s[r];
-    if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + h));
+    if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + (gate_elem ? h * Dv + e % Dv : h)));
     stf<T>(out + ((size_t)t * H + h) * Dv + e % Dv, o);
   }
 }
@@ -429,7 +454,7 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
 template <typename T>
 __global__ void __launch_bounds__(NT) attn_merge_kernel(const float* __restrict__ part, const T* __restrict__ gate,
                                                         int gate_ld, T* __restrict__ out, int H, int G, int Dv, int nsp,
-                                                        int nsplit, int rmax) {
+                                                        int nsplit, int rmax, int gate_elem) {
   const int t = blockIdx.x, g = blockIdx.y / nsp, r0 = (blockIdx.y % nsp) * rmax;
   const int R = min(rmax, H / G - r0), hq0 = g * (H / G) + r0, stride = rmax * (Dv + 2);
   const float* src = part + ((size_t)t * gridDim.y + blockIdx.y) * nsplit * stride;
@@ -445,7 +470,7 @@ __global__ void __launch_bounds__(NT) attn_merge_kernel(const float* __restrict_
       l += wz * src[z * stride + rmax * Dv + rmax + r];
     }
     float o = acc / l;
-    if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + hq0 + r));
+    if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + (gate_elem ? (hq0 + r) * Dv + e % Dv : hq0 + r)));
     stf<T>(out + ((size_t)t * H + hq0 + r) * Dv + e % Dv, o);
   }
 }
@@ -462,16 +487,26 @@ constexpr int MQ = 64, MK = 64;
 // RH query heads of one kv head per workgroup: a staged key / value tile serves all of them
 // (second launch bound: workgroups per CU the register budget must allow - four for 64-wide heads, so the
 // 1024 workgroups of a 4096-token, 16-head prompt are resident at once)
-// KVS: the value of a cached row is its first Dv numbers (a latent cache): the staged key tile serves as
-// the value tile, nothing is loaded twice
-template <int DK, int DV, int RH, bool KVS>
+// KVS: the value of a cached row is its first Dv numbers (a latent cache, or values that are the keys): the
+// staged key tile serves as the value tile, nothing is loaded twice
+// EXT: scores are capped (cap tanh(s / cap), cap > 0) and lose slopes[head] * distance; `window` is a chunk
+// size (a query sees its own chunk's start .. itself); sink[head] joins the softmax denominator; the gate
+// is [T, H * Dv], one per output coordinate
+struct AttnExt {
+  float scale, cap;
+  const float* slopes;
+  const float* sink;
+};
+
+template <int DK, int DV, int RH, bool KVS, bool EXT = false>
 __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1))) attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ gate, int gate_ld, const bf16_t* __restrict__ kp,
     const bf16_t* __restrict__ vp, const float* __restrict__ kb, const float* __restrict__ vb,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_len,
     const int* __restrict__ seq_off, const int* __restrict__ ptab, int ptab_ld, bf16_t* __restrict__ out, int n, int H,
-    int G, int PB, float scale_log2, int window, int pool, int kld, int vld) {
+    int G, int PB, float scale_log2, int window, int pool, int kld, int vld, AttnExt ext = AttnExt{}) {
   constexpr int D = 32 * DK, Dv = 16 * DV;
+  constexpr float LOG2E = 1.4426950408889634f;
   constexpr int KS = D * 2 + 16, VS = KVS ? KS : Dv * 2 + 16, PS = MK * 2 + 16;      // LDS row strides in bytes
   static_assert(!KVS || Dv <= D, "a value slice lies inside the key row");
   __shared__ __attribute__((aligned(16))) char k_lds[MK * KS];
@@ -513,8 +548,21 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
 #pragma unroll
     for (int i = 0; i < 4; ++i) { m_i[r][i] = -INFINITY; l_i[r][i] = 0.f; }
   }
+  float slope[RH];
+#pragma unroll
+  for (int r = 0; r < RH; ++r) slope[r] = 0.f;
+  if constexpr (EXT) {
+#pragma unroll
+    for (int r = 0; r < RH; ++r) {
+      if (ext.slopes) slope[r] = ext.slopes[h0 + r];
+      if (ext.sink) {                                        // the sink: a starting maximum with sum 1 and no value
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { m_i[r][i] = ext.sink[h0 + r] * LOG2E; l_i[r][i] = 1.f; }
+      }
+    }
+  }
   const int imin = start + qt * MQ, imax = start + min(len, qt * MQ + MQ) - 1;
-  const int jlo = window > 0 ? max(0, imin - window + 1) : 0;
+  const int jlo = window > 0 ? (EXT ? (imin / window) * window : max(0, imin - window + 1)) : 0;
   const int nbmax = (window > 0 && pool > 0 && imax - window + 1 > 0) ? (imax - window + 1) / pool : 0;
   const int tok_tiles = imax / MK - jlo / MK + 1, ntiles = tok_tiles + (nbmax + MK - 1) / MK;
   for (int i = tid; i < min(imax / MK + 1, NPID); i += NT) pid_s[i] = pt[i];
@@ -592,8 +640,20 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const int key = base + nt * 16 + c16;
-        const bool vis = tok ? (key <= qpos && (window <= 0 || qpos - key < window)) : key < seen;
-        const float v = vis ? sc[nt][i] * scale_log2 : -INFINITY;
+        bool vis;
+        float v;
+        if constexpr (EXT) {
+          vis = key <= qpos && (window <= 0 || key >= (qpos / window) * window);
+          float sv = sc[nt][i] * ext.scale;
+          if (ext.cap > 0.f) {                               // cap tanh(s / cap) = cap (1 - 2 / (e^(2 s / cap) + 1))
+            const float e2 = __builtin_amdgcn_exp2f(fminf(sv * (2.f * LOG2E / ext.cap), 126.f));
+            sv = ext.cap * (1.f - 2.f * __builtin_amdgcn_rcpf(e2 + 1.f));
+          }
+          v = vis ? (sv - slope[r] * (float)(qpos - key)) * LOG2E : -INFINITY;
+        } else {
+          vis = tok ? (key <= qpos && (window <= 0 || qpos - key < window)) : key < seen;
+          v = vis ? sc[nt][i] * scale_log2 : -INFINITY;
+        }
         sc[nt][i] = v;
         mx = fmaxf(mx, v);
       }
@@ -648,10 +708,17 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
 #pragma unroll
       for (int r = 0; r < RH; ++r) {
         float inv = l_i[r][i] > 0.f ? 1.f / l_i[r][i] : 0.f;
-        if (gate) inv *= sigmoidf_(bf2f(gate[(size_t)(off + t) * gate_ld + h0 + r]));
+        if constexpr (!EXT) {
+          if (gate) inv *= sigmoidf_(bf2f(gate[(size_t)(off + t) * gate_ld + h0 + r]));
+        }
 #pragma unroll
-        for (int dt = 0; dt < DV; ++dt)
-          out[((size_t)(off + t) * H + h0 + r) * Dv + dt * 16 + c16] = f2bf(o[r][dt][i] * inv);
+        for (int dt = 0; dt < DV; ++dt) {
+          float ov = o[r][dt][i] * inv;
+          if constexpr (EXT) {
+            if (gate) ov *= sigmoidf_(bf2f(gate[(size_t)(off + t) * gate_ld + (h0 + r) * Dv + dt * 16 + c16]));
+          }
+          out[((size_t)(off + t) * H + h0 + r) * Dv + dt * 16 + c16] = f2bf(ov);
+        }
       }
     }
   }
@@ -1126,7 +1193,7 @@ int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, co
 // nsplit > 1: the keys of every query are walked by nsplit workgroups (decode steps: few queries, long
 // windows); part = fp32 scratch [rows, G * nsp, nsplit, rmax * (Dv + 2)] (edge_sm_attention_part_floats)
 static size_t attn_lds_bytes(int rmax, int D, int Dv) {
-  return sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 3 * rmax) + sizeof(int) * KC;
+  return sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 4 * rmax) + sizeof(int) * KC;
 }
 
 // query heads of one kv head that share a workgroup: the whole group up to 16, fewer while their rows
@@ -1149,9 +1216,10 @@ size_t edge_sm_attention_part_floats(int rows, int H, int G, int D, int Dv, int 
 int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
-                      int window, int pool, int f32, int nsplit, float* part, int kld, int vld, hipStream_t st) {
+                      int window, int pool, int f32, int nsplit, float* part, int kld, int vld, int chunked, float cap,
+                      const float* slopes, const float* sink, int gate_elem, hipStream_t st) {
   if (rows == 0) return 0;
-  if (G <= 0 || H % G || Dv > 512) return -2;
+  if (G <= 0 || H % G || Dv > 512 || (chunked && pool > 0)) return -2;
   const int R = H / G;
   const int rmax = edge_sm_attention_rmax(rows, H, G, D, Dv);
   if (rmax == 0) return -3;
@@ -1163,7 +1231,7 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
   SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL, V>), dim3(rows, G * nsp, nsplit), dim3(NT), lds, st, (const T*)q,         \
                                (const T*)gate, gate_ld, (const T*)kp, (const T*)vp, kb, vb, tok_seq, tok_pos,       \
                                seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool, nsp, nsplit, part, \
-                               kld, vld))
+                               kld, vld, chunked, cap, slopes, sink, gate_elem))
 #define SM_ATT(RM, DL)               \
   do {                               \
     if (vec) SM_ATT_V(RM, DL, true); \
@@ -1186,7 +1254,7 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
 #undef SM_ATT_V
   if (nsplit > 1)
     SM_T(f32, hipLaunchKernelGGL(attn_merge_kernel<T>, dim3(rows, G * nsp), dim3(NT), 0, st, part, (const T*)gate, gate_ld,
-                                 (T*)out, H, G, Dv, nsp, nsplit, rmax));
+                                 (T*)out, H, G, Dv, nsp, nsplit, rmax, gate_elem));
   return (int)hipGetLastError();
 }
 
@@ -1257,8 +1325,10 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
                            const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
                            const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
                            int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
-                           int pool, int kld, int vld, hipStream_t st) {
+                           int pool, int kld, int vld, int chunked, float cap, const float* slopes, const float* sink,
+                           int gate_elem, hipStream_t st) {
   if (page != MK || G <= 0 || H % G || kld % 8 || vld % 8) return 1;
+  const bool extras = chunked || cap > 0.f || slopes || sink || gate_elem;
   if (n == 0 || qtiles == 0) return 0;
   const float sl2 = scale * 1.4426950408889634f;
   // query heads per workgroup: a staged tile can serve 4 or 2 heads of a kv group, but the kernel is
@@ -1271,6 +1341,31 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
   else if (R % 2 == 0 && (long)qtiles * (H / 2) >= 1024) rh = 2;
   const bool kvs = kp == vp && kld == vld;
   if (kvs && pool > 0) return 1;                             // pooled entries keep separate key / value rows
+  if (extras) {
+    // the capped / biased / chunked form: values that are the keys, an element-wise gate or none
+    if (!kvs || D != Dv || pool > 0 || (window > 0 && !chunked) || (gate && !gate_elem)) return 1;
+    const AttnExt ext{scale, cap, slopes, sink};
+#define SM_MFX_R(DK, DV, RH)                                                                                         \
+  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV, RH, true, true>), dim3(qtiles, H / RH), dim3(NT), 0, st,              \
+                     (const bf16_t*)q, (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb,   \
+                     seq_slot, seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window,   \
+                     pool, kld, vld, ext)
+#define SM_MFX(DK, DV)                    \
+  do {                                    \
+    if (rh == 4) SM_MFX_R(DK, DV, 4);     \
+    else if (rh == 2) SM_MFX_R(DK, DV, 2);\
+    else SM_MFX_R(DK, DV, 1);             \
+  } while (0)
+    if (D == 32) SM_MFX(1, 2);
+    else if (D == 64) SM_MFX(2, 4);
+    else if (D == 96) SM_MFX(3, 6);
+    else if (D == 128) SM_MFX(4, 8);
+    else if (D == 256) SM_MFX_R(8, 16, 1);
+    else return 1;
+#undef SM_MFX
+#undef SM_MFX_R
+    return (int)hipGetLastError();
+  }
 #define SM_MF_ARGS                                                                                                  \
   dim3(NT), 0, st, (const bf16_t*)q, (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb,     \
       seq_slot, seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window, pool, kld, vld

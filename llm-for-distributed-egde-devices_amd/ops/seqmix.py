@@ -188,10 +188,12 @@ def _rotate_half(x, cs, dims):
 
 
 def rope_paged_write(proj: torch.Tensor, meta: RaggedMeta, rope: Optional[torch.Tensor], k_pages: torch.Tensor,
-                     v_pages: torch.Tensor, heads: int, rot_dims: int) -> torch.Tensor:
+                     v_pages: Optional[torch.Tensor], heads: int, rot_dims: int) -> torch.Tensor:
     """proj [T, q | k | v | ...] -> rotated q [T, heads, D]; the rotated keys and the values go
-    to their pages ``[pages, page, kv heads, D | Dv]`` at each token's position."""
-    G, D, Dv = k_pages.shape[2], k_pages.shape[3], v_pages.shape[3]
+    to their pages ``[pages, page, kv heads, D | Dv]`` at each token's position.  ``v_pages`` None:
+    proj is [T, q | k] and only keys are cached (a layer whose values are its keys)."""
+    G, D = k_pages.shape[2], k_pages.shape[3]
+    Dv = v_pages.shape[3] if v_pages is not None else 0
     if _gpu(proj):
         return _ext().sm_rope_write(proj, meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.page_table,
                                     rope if rot_dims else None, k_pages, v_pages, int(heads), int(rot_dims))
@@ -207,7 +209,8 @@ def rope_paged_write(proj: torch.Tensor, meta: RaggedMeta, rope: Optional[torch.
     slot = meta.seq_slot.long()[meta.tok_seq.long()]
     pid = meta.page_table[slot, pos // meta.page].long()
     k_pages[pid, pos % meta.page] = k.to(k_pages.dtype)
-    v_pages[pid, pos % meta.page] = v.to(v_pages.dtype)
+    if v_pages is not None:
+        v_pages[pid, pos % meta.page] = v.to(v_pages.dtype)
     return q.to(proj.dtype)
 
 
@@ -251,7 +254,8 @@ def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages
         return _ext().sm_attention(q, gate, k_pages, v_pages, k_pool if pool else None, v_pool if pool else None,
                                    meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.page_table, float(scale),
                                    int(window) if window is not None else 0, int(pool or 0), int(meta.max_keys),
-                                   meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n), int(qtiles))
+                                   meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n), int(qtiles), False, 0.0,
+                                   None, None)
     page = meta.page
     out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
     R = H // G
@@ -287,6 +291,59 @@ def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[..., None]
     return out.reshape(T, H * Dv).to(q.dtype)
+
+
+def distance_slopes(heads: int, device=None) -> torch.Tensor:
+    """fp32 [heads]: slope_h = 2^(-8 (h + 1) / heads), the rate at which head h's scores fall with distance."""
+    h = torch.arange(1, heads + 1, dtype=torch.float64)
+    return torch.pow(2.0, -8.0 * h / heads).to(torch.float32).to(device)
+
+
+def chunk_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages: torch.Tensor, meta: RaggedMeta, scale: float,
+                    chunk: Optional[int], softcap: Optional[float], slopes: Optional[torch.Tensor],
+                    sink: Optional[torch.Tensor]) -> torch.Tensor:
+    """q [T, H, D] -> [T, H * D] over cached keys that are also the values.  Query position i sees
+    j <= i with floor(i / chunk) == floor(j / chunk) (``chunk`` None: every j <= i).  Scores in fp32:
+    s = (q . k) scale; s <- softcap tanh(s / softcap) (``softcap`` None: as is); s <- s - slopes[h] (i - j)
+    (``slopes`` fp32 [H] or None).  The softmax denominator also holds exp(sink[h]) (``sink`` fp32 [H] or
+    None), which has no value.  ``gate`` ([T, H * D] view): the result times sigmoid(gate), element by element."""
+    T, H, D = q.shape
+    G = k_pages.shape[2]
+    if _gpu(q):
+        qtiles = 0
+        if q.dtype == torch.bfloat16 and meta.max_len >= ATTN_MFMA_MIN:
+            qtiles = sum((h[2] + 63) // 64 for h in meta.host)
+        return _ext().sm_attention(q, gate, k_pages, k_pages, None, None, meta.tok_seq, meta.tok_pos, meta.seq_slot,
+                                   meta.page_table, float(scale), int(chunk or 0), 0, int(meta.max_keys), meta.seq_start,
+                                   meta.seq_len, meta.seq_off, int(meta.n), int(qtiles), True, float(softcap or 0.0),
+                                   slopes, sink)
+    page, R = meta.page, H // G
+    out = torch.empty(T, H, D, dtype=torch.float32, device=q.device)
+    for slot, start, n, off in meta.host:
+        L = start + n
+        pos = torch.arange(L, device=q.device)
+        pid = meta.page_table[slot, pos // page].long()
+        k = k_pages[pid, pos % page].float()                     # [L, G, D]
+        qi = q[off:off + n].float().view(n, G, R, D)
+        i = torch.arange(start, L, device=q.device)
+        s = torch.einsum("ngrd,lgd->ngrl", qi, k) * scale
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
+        d = (i[:, None] - pos[None])
+        if slopes is not None:
+            s = s - slopes.float().view(1, G, R, 1) * d[:, None, None, :].float()
+        vis = d >= 0
+        if chunk:
+            vis &= (i[:, None] // chunk) == (pos[None] // chunk)
+        s = s.masked_fill(~vis[:, None, None, :], float("-inf"))
+        if sink is not None:
+            s = torch.cat([s, sink.float().view(1, G, R, 1).expand(n, G, R, 1)], -1)
+        p = torch.softmax(s, -1)[..., :L]
+        out[off:off + n] = torch.einsum("ngrl,lgd->ngrd", p, k).reshape(n, H, D)
+    out = out.reshape(T, H * D)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(q.dtype)
 
 
 # --------------------------------------------------------------------------- state-space side
@@ -420,6 +477,36 @@ def layer_norm_residual(x: torch.Tensor, y: Optional[torch.Tensor], weight: torc
     return x
 
 
+def _group_rms(v: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
+    T, W = v.shape
+    g = v.view(T, groups, W // groups)
+    return (g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)).view(T, W)
+
+
+def group_rms_norm(x: torch.Tensor, weight: torch.Tensor, groups: int, eps: float, out_dtype) -> torch.Tensor:
+    """RMS norm in ``groups`` equal consecutive parts of fp32 rows [T, W] (each part over its own
+    sqrt(mean^2 + eps)), the whole times weight [W], stored as ``out_dtype``."""
+    if _gpu(x):
+        return _ext().sm_group_norm(x, weight, int(groups), float(eps), out_dtype == torch.float32)
+    return (_group_rms(x.float(), groups, eps) * weight.float()).to(out_dtype)
+
+
+def group_norm_residual(x: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor, groups: int, eps: float,
+                        mult: float, parts: Optional[torch.Tensor] = None,
+                        part_w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x (fp32 [T, W], in place) += mult * group-RMS-norm(v) weight, with v = y + sum_k part_w[:, k]
+    parts[:, k] summed in fp32 in k order (``y`` None: the parts alone; ``part_w`` None: ones)."""
+    if _gpu(x):
+        _ext().sm_group_norm_residual(x, y, weight, int(groups), float(eps), float(mult), parts, part_w)
+        return x
+    v = y.float() if y is not None else torch.zeros_like(x)
+    if parts is not None:
+        for k in range(parts.shape[1]):
+            v = v + (parts[:, k].float() if part_w is None else part_w[:, k:k + 1] * parts[:, k].float())
+    x.add_(_group_rms(v, groups, eps) * weight.float(), alpha=mult)
+    return x
+
+
 def rms_norm_cols(u: torch.Tensor, c0: int, C: int, weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
     """RMS norm (fp32) of columns [c0, c0 + C) of u [T, *] times weight [C], contiguous ``out_dtype``."""
     if _gpu(u):
@@ -436,6 +523,17 @@ def glu_clamp(u: torch.Tensor, ff: int, limit: float) -> torch.Tensor:
     g = u[:, :ff].float().clamp(max=limit)
     up = u[:, ff:2 * ff].float().clamp(-limit, limit)
     return (g * torch.sigmoid(1.702 * g) * (up + 1)).to(u.dtype)
+
+
+def glu_silu(u: torch.Tensor, ff: int, row_w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """u [T, gate | up] -> silu(w gate) (w up) with w = row_w[t] (fp32 [T]; None: 1): the gated unit of
+    an input scaled by w, computed from the unscaled projections (fp32 math, stored in u's dtype)."""
+    if _gpu(u):
+        return _ext().sm_glu_silu(u, int(ff), row_w)
+    g, up = u[:, :ff].float(), u[:, ff:2 * ff].float()
+    if row_w is not None:
+        g, up = g * row_w[:, None], up * row_w[:, None]
+    return (F.silu(g) * up).to(u.dtype)
 
 
 # --------------------------------------------------------------------------- latent attention
@@ -500,9 +598,27 @@ def delta_prepare(qkv: torch.Tensor, u: torch.Tensor, b0: int, a: torch.Tensor, 
     return torch.cat([q.reshape(T, GN), k.reshape(T, GN), g.reshape(T, heads * N), beta], -1)
 
 
+def delta_prepare_head(qkv: torch.Tensor, u: torch.Tensor, b0: int, a0: int, dt_bias: torch.Tensor,
+                       A_log: torch.Tensor, heads: int, kv_heads: int, N: int):
+    """``delta_prepare`` for one decay per head: the decay of head h is
+    exp(-exp(A_log[h]) softplus(u[:, a0 + h] + dt_bias[h])), beta = sigmoid of columns [b0, b0 + heads)
+    of u.  Returns fp32 [T, 2 kv_heads N + 2 heads]: q | k | decay | beta."""
+    if _gpu(qkv):
+        return _ext().sm_delta_prep_head(qkv, u, int(b0), int(a0), dt_bias, A_log, int(heads), int(kv_heads), int(N))
+    T, GN = qkv.shape[0], kv_heads * N
+    unit = lambda x: x * torch.rsqrt(x.pow(2).sum(-1, keepdim=True) + 1e-6)
+    q = unit(qkv[:, :GN].float().view(T, kv_heads, N)) * N ** -0.5
+    k = unit(qkv[:, GN:2 * GN].float().view(T, kv_heads, N))
+    sp = F.softplus(u[:, a0:a0 + heads].float() + dt_bias.float(), threshold=1e9)
+    g = torch.exp(-torch.exp(A_log.float())[None] * sp)
+    beta = torch.sigmoid(u[:, b0:b0 + heads].float())
+    return torch.cat([q.reshape(T, GN), k.reshape(T, GN), g, beta], -1)
+
+
 def delta_rule_scan(prep: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, meta: RaggedMeta, heads: int,
                     kv_heads: int, N: int, P: int) -> torch.Tensor:
-    """The gated delta rule, token by token in fp32.  ``prep`` from ``delta_prepare``; the values are
+    """The gated delta rule, token by token in fp32.  ``prep`` from ``delta_prepare`` (a decay per
+    head and key channel) or ``delta_prepare_head`` (one per head: the row is shorter); the values are
     columns [2 kv_heads N, ..) of ``qkv``.  Per head, with S [N, P]:  S <- g * S (rows) ;
     w = beta (v - S^T k) ;  S <- S + k w^T ;  o = S^T q.  state [slots, heads, N, P] fp32 is read
     (zero for a portion starting at 0) and left at the portion's end.  Returns o fp32 [T, heads P]."""
@@ -510,6 +626,9 @@ def delta_rule_scan(prep: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, 
         return _ext().sm_delta_scan(prep, qkv, state, meta.seq_slot, meta.seq_start, meta.seq_len, meta.seq_off,
                                     int(meta.n), int(heads), int(kv_heads), int(N), int(P))
     T, GN, rep = prep.shape[0], kv_heads * N, heads // kv_heads
+    if prep.shape[1] == 2 * GN + 2 * heads and N != 1:           # per-head decays: one number for all key channels
+        prep = torch.cat([prep[:, :2 * GN], prep[:, 2 * GN:2 * GN + heads].repeat_interleave(N, 1),
+                          prep[:, 2 * GN + heads:]], -1)
     out = torch.empty(T, heads * P, dtype=torch.float32, device=prep.device)
     for slot, start, n, off in meta.host:
         pr = prep[off:off + n]
@@ -528,25 +647,32 @@ def delta_rule_scan(prep: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, 
     return out
 
 
-def head_norm_gate(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, heads: int, eps: float, out_dtype) -> torch.Tensor:
+def head_norm_gate(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, heads: int, eps: float, out_dtype,
+                   act: str = "sigmoid") -> torch.Tensor:
     """Each head's part of y (fp32 [T, heads P]) divided by its root mean square, times weight [P]
-    (shared by the heads), times sigmoid(z) (z [T, heads P], a possibly strided view)."""
+    (shared by the heads), times sigmoid(z) or silu(z) (``act``; z [T, heads P], a possibly strided view)."""
     if _gpu(y):
-        return _ext().sm_head_norm_gate(y, z, weight, int(heads), float(eps), out_dtype == torch.float32)
+        return _ext().sm_head_norm_gate(y, z, weight, int(heads), float(eps), out_dtype == torch.float32, act == "silu")
     T, C = y.shape
     g = y.view(T, heads, C // heads)
     g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
-    return (g.view(T, C) * torch.sigmoid(z.float())).to(out_dtype)
+    gate = F.silu(z.float()) if act == "silu" else torch.sigmoid(z.float())
+    return (g.view(T, C) * gate).to(out_dtype)
 
 
 # --------------------------------------------------------------------------- mixture of experts
-def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float):
-    """Softmax router in fp32 over h [T, W] (router fp32 [E, W]): the ``top`` largest scores of every
-    token, divided by their sum (+ 1e-20) and multiplied by ``scale``.  Returns (expert ids int32
-    [T, top], weights fp32 [T, top]), largest first."""
+def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, mode: str = "softmax"):
+    """Router in fp32 over h [T, W] (router fp32 [E, W]).  ``mode`` "softmax": the ``top`` largest
+    softmax scores of every token, divided by their sum (+ 1e-20) and multiplied by ``scale``;
+    "sigmoid": the ``top`` largest of sigmoid(logit) as they are, times ``scale``.  Returns (expert ids
+    int32 [T, top], weights fp32 [T, top]), largest first (the lower id on a tie)."""
     if _gpu(h):
-        return _ext().sm_moe_route(h, router, int(top), float(scale))
-    s = torch.softmax(h.float() @ router.float().t(), -1)
+        return _ext().sm_moe_route(h, router, int(top), float(scale), mode == "sigmoid")
+    z = h.float() @ router.float().t()
+    if mode == "sigmoid":
+        w, idx = torch.topk(torch.sigmoid(z), top, -1)
+        return idx.int(), w * scale
+    s = torch.softmax(z, -1)
     w, idx = torch.topk(s, top, -1)
     return idx.int(), w / (w.sum(-1, keepdim=True) + 1e-20) * scale
 
@@ -554,24 +680,31 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float):
 MOE_GEMM_MIN = int(__import__("os").environ.get("EDGELLM_MOE_GEMM_MIN", "64"))
 
 
-def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, limit: float) -> torch.Tensor:
+def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, limit: float,
+                act: str = "glu_clamp", in_w: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Every token's chosen experts: h [T, W], idx int32 [T, top], w_gu [E, 2 ff, W] (gate rows, then
-    up rows), w_down [E, W, ff] -> the experts' outputs [T, top, W] (not yet weighted)."""
+    up rows), w_down [E, W, ff] -> the experts' outputs [T, top, W] (not yet weighted).  ``act``
+    "glu_clamp" (with ``limit``) or "silu_glu"; ``in_w`` fp32 [T, top] (silu_glu only): choice k runs on
+    in_w[t, k] h[t] (the experts have no biases, so the weight is applied to the gate and up
+    projections' outputs in fp32)."""
     T, top = idx.shape
     E, ff2, W = w_gu.shape
+    assert act in ("glu_clamp", "silu_glu") and (in_w is None or act == "silu_glu")
     if _gpu(h):
         if T >= MOE_GEMM_MIN:
-            return _moe_experts_sorted(h, idx, w_gu, w_down, limit)
-        return _ext().sm_moe_experts(h, idx, w_gu, w_down, float(limit))
+            return _moe_experts_sorted(h, idx, w_gu, w_down, limit, act, in_w)
+        return _ext().sm_moe_experts(h, idx, w_gu, w_down, float(limit), act == "silu_glu", in_w)
     out = torch.zeros(T, top, w_down.shape[1], dtype=h.dtype, device=h.device)
     for e in idx.unique().tolist():
         t, k = (idx == e).nonzero(as_tuple=True)
-        y = glu_clamp(F.linear(h[t], w_gu[e]), ff2 // 2, limit)
+        u = F.linear(h[t], w_gu[e])
+        y = glu_clamp(u, ff2 // 2, limit) if act == "glu_clamp" else \
+            glu_silu(u, ff2 // 2, None if in_w is None else in_w[t, k])
         out[t, k] = F.linear(y, w_down[e])
     return out
 
 
-def _moe_experts_sorted(h, idx, w_gu, w_down, limit):
+def _moe_experts_sorted(h, idx, w_gu, w_down, limit, act="glu_clamp", in_w=None):
     """Prompt-sized steps: (token, choice) pairs sorted by expert; every expert's rows run through its
     gate | up weights, one activation launch covers all rows, every expert's rows run through its down
     weights, and the rows go back to (token, choice) order.  bf16 on the GPU: the library's grouped
@@ -583,9 +716,11 @@ def _moe_experts_sorted(h, idx, w_gu, w_down, limit):
     order = torch.argsort(flat, stable=True)
     counts = torch.bincount(flat, minlength=E)
     rows = h.index_select(0, order // top)
+    row_w = in_w.reshape(-1).index_select(0, order) if in_w is not None else None
+    glu = (lambda u_: glu_clamp(u_, ff2 // 2, limit)) if act == "glu_clamp" else (lambda u_: glu_silu(u_, ff2 // 2, row_w))
     if h.is_cuda and h.dtype == torch.bfloat16 and W % 8 == 0 and ff2 % 16 == 0 and hasattr(torch, "_grouped_mm"):
         ends = torch.cumsum(counts, 0).to(torch.int32)
-        y = glu_clamp(torch._grouped_mm(rows, w_gu.transpose(1, 2), offs=ends), ff2 // 2, limit)
+        y = glu(torch._grouped_mm(rows, w_gu.transpose(1, 2), offs=ends))
         o = torch._grouped_mm(y, w_down.transpose(1, 2), offs=ends)
     else:
         u = torch.empty(T * top, ff2, dtype=h.dtype, device=h.device)
@@ -596,7 +731,7 @@ def _moe_experts_sorted(h, idx, w_gu, w_down, limit):
                 spans.append((e, a, n))
                 torch.mm(rows[a:a + n], w_gu[e].t(), out=u[a:a + n])
                 a += n
-        y = glu_clamp(u, ff2 // 2, limit)
+        y = glu(u)
         for e, a, n in spans:
             torch.mm(y[a:a + n], w_down[e].t(), out=o[a:a + n])
     back = torch.empty_like(order)
