@@ -84,29 +84,38 @@ def delta_mixer(h, p, m, eps):
     return (o * gate).reshape(L, H * P) @ f64(p["o"]).T
 
 
-def chunk_attention(h, p, m):
-    """Chunked causal attention with tanh-capped scores, a linear distance bias, a sink in the
-    softmax denominator, values = keys, and a sigmoid output gate."""
-    H, G, D = m["heads"], m["kv_heads"], m["dim"]
-    L = h.shape[0]
-    scale, cap = float(m["scale"]), m.get("softcap")
-    chunk = (m.get("mask") or {}).get("size")
-    q = (h @ f64(p["q"]).T).reshape(L, H, D)
-    k = (h @ f64(p["k"]).T).reshape(L, G, D)
-    sink = f64(p["sink"])
+def attention_core(q, k, scale, cap, chunk, sink, biased=True):
+    """q [L, H, D], k [L, G, D] -> [L, H, D]: for query i the keys j <= i of its own chunk
+    (floor(i / chunk) == floor(j / chunk); chunk None: all j <= i); score (q . k) scale, capped as
+    cap tanh(score / cap), minus 2^(-8 (h + 1) / H) (i - j); exp(sink_h) joins the denominator only;
+    the output is the weighted sum of the keys themselves."""
+    L, H, D = q.shape
+    G = k.shape[1]
     out = np.zeros((L, H, D))
     for hd in range(H):
         kv = hd // (H // G)
-        slope = 2.0 ** (-8.0 * (hd + 1) / H)
+        slope = 2.0 ** (-8.0 * (hd + 1) / H) if biased else 0.0
         for i in range(L):
             lo = (i // chunk) * chunk if chunk else 0
             s = (k[lo:i + 1, kv] @ q[i, hd]) * scale
             if cap:
                 s = cap * np.tanh(s / cap)
             s = s - slope * (i - np.arange(lo, i + 1))
-            mx = max(s.max(), sink[hd])
+            mx = s.max() if sink is None else max(s.max(), sink[hd])
             e = np.exp(s - mx)
-            out[i, hd] = (e @ k[lo:i + 1, kv]) / (e.sum() + math.exp(sink[hd] - mx))
+            den = e.sum() + (0.0 if sink is None else math.exp(sink[hd] - mx))
+            out[i, hd] = (e @ k[lo:i + 1, kv]) / den
+    return out
+
+
+def chunk_attention(h, p, m):
+    """Chunked causal attention with tanh-capped scores, a linear distance bias, a sink in the
+    softmax denominator, values = keys, and a sigmoid output gate."""
+    H, G, D = m["heads"], m["kv_heads"], m["dim"]
+    L = h.shape[0]
+    q = (h @ f64(p["q"]).T).reshape(L, H, D)
+    k = (h @ f64(p["k"]).T).reshape(L, G, D)
+    out = attention_core(q, k, float(m["scale"]), m.get("softcap"), (m.get("mask") or {}).get("size"), f64(p["sink"]))
     gate = sigmoid(h @ f64(p["g"]).T)
     return (out.reshape(L, H * D) * gate) @ f64(p["o"]).T
 
