@@ -2,7 +2,10 @@
 (``bench.py --hybrid-compare``): the Nudadra hybrid beside the parallel-residual row-cache decoder,
 or (``--hybrid-family pagonex``) the Pagonex model (latent attention and gated delta-rule layers,
 mixture-of-experts feed-forwards) beside the Nudadra hybrid, its closest relative: the same engine,
-windowed attention over the paged cache, a recurrent mixer and a feed-forward per layer.
+windowed attention over the paged cache, a recurrent mixer and a feed-forward per layer; or
+(``--hybrid-family vetevik``) the Vetevik model (chunked attention whose values are its keys, a gated
+delta rule with per-head decays, sigmoid-routed experts, norms on both sides of every sublayer)
+beside the Pagonex model of equal width, heads, state size and active expert width.
 
 Sizes resemble real layers (random weights): the hybrid layer has windowed attention with pooled
 blocks + a Mamba-2 mixer + a squared-ReLU feed-forward; the comparison model is the
@@ -21,8 +24,8 @@ from typing import Dict, List
 
 import torch
 
-from ..models.configs import (DeltaSpec, LatentAttnSpec, LayerSpec, ModelConfig, MoESpec, SSDSpec, WindowAttnSpec,
-                              PRESETS)
+from ..models.configs import (ChunkAttnSpec, DeltaSpec, LatentAttnSpec, LayerSpec, ModelConfig, MoESpec, SSDSpec,
+                              WindowAttnSpec, PRESETS)
 from ..models.decoder import build_model
 from ..models.hybrid import build_hybrid
 from .generate import Generator, SamplingParams
@@ -82,6 +85,34 @@ def pagonex_config(s: dict) -> ModelConfig:
                        logit_scale=1.0)
 
 
+# Vetevik sizes: attention and delta-rule layers alternate as in the Pagonex size of the same name, with its
+# width, head count, head sizes, state size and expert width; four experts per token make the active
+# feed-forward width equal to Pagonex's three + shared; the chunk is as long as Pagonex's window
+VETEVIK_SIZES = {
+    "w1024": dict(width=1024, layers=4, heads=16, kv=4, dim=64, chunk=512, softcap=50.0, d_heads=16, d_dim=64, d_vdim=64,
+                  experts=16, top=4, ff=1024, groups=2, vocab=32000),
+    "w2048": dict(width=2048, layers=4, heads=16, kv=4, dim=128, chunk=1024, softcap=50.0, d_heads=16, d_dim=128,
+                  d_vdim=128, experts=32, top=4, ff=2048, groups=2, vocab=32000),
+}
+
+
+def vetevik_config(s: dict) -> ModelConfig:
+    moe = MoESpec(s["experts"], s["top"], 1.0, s["ff"], router="sigmoid", act="silu_glu", weight_on="input")
+    specs = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            a = ChunkAttnSpec(s["heads"], s["kv"], s["dim"], s["dim"] ** -0.5, s["chunk"], s["softcap"])
+            specs.append(LayerSpec("chunk_attention", chunk_attn=a, moe=moe))
+        else:
+            d = DeltaSpec(s["d_heads"], s["d_heads"], s["d_dim"], s["d_vdim"], 4, decay="head")
+            specs.append(LayerSpec("head_delta", delta=d, moe=moe))
+    return ModelConfig(arch="vetevik", vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
+                       num_heads=s["heads"], num_kv_heads=s["kv"], intermediate_size=0, head_dim=s["dim"],
+                       max_position_embeddings=1 << 20, norm="rms_group", norm_eps=1e-6, act="silu_glu", pos_emb="none",
+                       tie_word_embeddings=True, name="vetevik-bench", layer_specs=specs, norm_groups=s["groups"],
+                       residual_mult=0.3)
+
+
 def closest_config(s: dict) -> ModelConfig:
     return PRESETS["phi-2"].replace(vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
                                     num_heads=s["heads"], num_kv_heads=s["kv"], head_dim=s["dim"], rotary_dim=s["dim"],
@@ -130,7 +161,8 @@ def op_times(eng: RaggedEngine, entries, close=()) -> Dict[str, float]:
     names = ["embedding_scaled", "scalar_rms_norm", "relu2", "cat_cast", "combine_residual", "gated_group_norm",
              "rope_paged_write", "pool_blocks", "window_pool_attention", "conv_silu", "ssd_scan", "linear_f32",
              "embedding_bigram", "canon_conv", "layer_norm_rows", "layer_norm_residual", "rms_norm_cols", "glu_clamp",
-             "latent_write", "delta_prepare", "delta_rule_scan", "head_norm_gate", "moe_route", "moe_experts"]
+             "latent_write", "delta_prepare", "delta_rule_scan", "head_norm_gate", "moe_route", "moe_experts",
+             "group_rms_norm", "group_norm_residual", "chunk_attention", "delta_prepare_head"]
     saved = {n: getattr(seqmix, n) for n in names}
     lin = F.linear
 
@@ -207,10 +239,29 @@ def run_pagonex(sizes: List[str], prompt: int, batch: int, steps: int, device) -
             "decode_batch": batch, "decode_steps": steps, "sizes": res}
 
 
+def run_vetevik(sizes: List[str], prompt: int, batch: int, steps: int, device) -> Dict:
+    res = {}
+    r2 = lambda d: {k: (round(v, 2) if isinstance(v, float) else v) for k, v in d.items()}
+    for name in sizes:
+        s, c = VETEVIK_SIZES[name], PAGONEX_SIZES[name]
+        v = bench_hybrid(s, prompt, batch, steps, device, vetevik_config(s))
+        torch.cuda.empty_cache()
+        p = bench_hybrid(c, prompt, batch, steps, device, pagonex_config(c))
+        torch.cuda.empty_cache()
+        res[name] = {"size": s, "closest_size": c, "vetevik": r2(v), "closest_pagonex": r2(p),
+                     "prefill_ratio": round(v["prefill_tok_s"] / p["prefill_tok_s"], 3),
+                     "decode_ratio": round(v["decode_tok_s"] / p["decode_tok_s"], 3)}
+    return {"metric": "prefill / decode tokens/s, Vetevik layer-spec model vs the Pagonex model of equal size",
+            "dtype": "bf16", "data": "synthetic (random weights, random prompt)", "prompt_tokens": prompt,
+            "decode_batch": batch, "decode_steps": steps, "sizes": res}
+
+
 def run(sizes: List[str], prompt: int = 4096, batch: int = 4, steps: int = 32, device=None, family: str = "nudadra") -> Dict:
     device = torch.device(device or "cuda:0")
     if family == "pagonex":
         return run_pagonex(sizes, prompt, batch, steps, device)
+    if family == "vetevik":
+        return run_vetevik(sizes, prompt, batch, steps, device)
     res = {}
     for name in sizes:
         s = SIZES[name]

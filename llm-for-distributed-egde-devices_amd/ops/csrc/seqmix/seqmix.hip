@@ -548,13 +548,23 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
 #pragma unroll
     for (int i = 0; i < 4; ++i) { m_i[r][i] = -INFINITY; l_i[r][i] = 0.f; }
   }
-  float slope[RH];
+  // EXT: a score in the log2 domain is c1 - c2 / (2^(xs s) + 1) - sl2 (i - j)  (cap tanh(x / cap) written with one
+  // exp2 and one rcp; no cap: s scale_log2 - sl2 (i - j)); clo = first position of each row's chunk
+  float sl2[RH];
+  int clo[4];
+  const float c1 = ext.cap * LOG2E, c2 = 2.f * ext.cap * LOG2E, xs = ext.cap > 0.f ? ext.scale * 2.f * LOG2E / ext.cap : 0.f;
 #pragma unroll
-  for (int r = 0; r < RH; ++r) slope[r] = 0.f;
+  for (int r = 0; r < RH; ++r) sl2[r] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) clo[i] = 0;
   if constexpr (EXT) {
+    if (window > 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) clo[i] = ((start + wq0 + 4 * g4 + i) / window) * window;
+    }
 #pragma unroll
     for (int r = 0; r < RH; ++r) {
-      if (ext.slopes) slope[r] = ext.slopes[h0 + r];
+      if (ext.slopes) sl2[r] = ext.slopes[h0 + r] * LOG2E;
       if (ext.sink) {                                        // the sink: a starting maximum with sum 1 and no value
 #pragma unroll
         for (int i = 0; i < 4; ++i) { m_i[r][i] = ext.sink[h0 + r] * LOG2E; l_i[r][i] = 1.f; }
@@ -643,13 +653,13 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
         bool vis;
         float v;
         if constexpr (EXT) {
-          vis = key <= qpos && (window <= 0 || key >= (qpos / window) * window);
-          float sv = sc[nt][i] * ext.scale;
-          if (ext.cap > 0.f) {                               // cap tanh(s / cap) = cap (1 - 2 / (e^(2 s / cap) + 1))
-            const float e2 = __builtin_amdgcn_exp2f(fminf(sv * (2.f * LOG2E / ext.cap), 126.f));
-            sv = ext.cap * (1.f - 2.f * __builtin_amdgcn_rcpf(e2 + 1.f));
-          }
-          v = vis ? (sv - slope[r] * (float)(qpos - key)) * LOG2E : -INFINITY;
+          vis = key <= qpos && key >= clo[i];
+          const float bias = sl2[r] * (float)(qpos - key);
+          if (ext.cap > 0.f)                                 // 2^(xs s) = inf gives the cap itself, 0 gives -cap
+            v = c1 - c2 * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(sc[nt][i] * xs) + 1.f) - bias;
+          else
+            v = sc[nt][i] * scale_log2 - bias;
+          v = vis ? v : -INFINITY;
         } else {
           vis = tok ? (key <= qpos && (window <= 0 || qpos - key < window)) : key < seen;
           v = vis ? sc[nt][i] * scale_log2 : -INFINITY;
