@@ -406,7 +406,8 @@ __global__ void __launch_bounds__(NT) moe_logits_kernel(const T* __restrict__ h,
 
 // One wave per token: softmax over the experts' scores, then the `top` largest (lowest index on a tie),
 // divided by their sum (+ 1e-20) and multiplied by scale.  sigm: the scores are sigmoid(z) and the `top`
-// largest keep their own value (times scale).
+// largest keep their own value (times scale); they are picked by z itself (the same order), so scores that
+// round to 1 do not tie.
 __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ z, int E, int top, float scale,
                                                       int* __restrict__ idx, float* __restrict__ wts, int sigm) {
   extern __shared__ __attribute__((aligned(16))) float z_s[];   // [E]
@@ -415,9 +416,7 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
   float mx = -INFINITY;
   for (int e = lane; e < E; e += 64) { z_s[e] = z[t * E + e]; mx = fmaxf(mx, z_s[e]); }
   mx = wave_max(mx);
-  if (sigm) {
-    for (int e = lane; e < E; e += 64) z_s[e] = sigmoidf_(z_s[e]);
-  } else {
+  if (!sigm) {
     float sum = 0.f;
     for (int e = lane; e < E; e += 64) sum += expf(z_s[e] - mx);
     sum = wave_sum(sum);
@@ -425,8 +424,9 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
   }
   float tot = 0.f, my_w = 0.f;
   int my_i = 0;                                              // lane k keeps the k-th choice
+  const float gone = sigm ? -INFINITY : -2.f;                // what a taken entry becomes (below every live one)
   for (int k = 0; k < top; ++k) {
-    float best = -1.f;
+    float best = sigm ? -INFINITY : -1.f;
     int bi = E;
     for (int e = lane; e < E; e += 64)
       if (z_s[e] > best) { best = z_s[e]; bi = e; }
@@ -441,12 +441,12 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
       best = 0.f;
     }
     if (lane == k) { my_w = best; my_i = bi; }
-    if (lane == 0) z_s[bi] = -2.f;                           // LDS accesses of one wave keep their order
+    if (lane == 0) z_s[bi] = gone;                           // LDS accesses of one wave keep their order
     tot += best;
   }
   if (lane < top) {
     idx[t * top + lane] = my_i;
-    wts[t * top + lane] = sigm ? my_w * scale : my_w / (tot + 1e-20f) * scale;
+    wts[t * top + lane] = sigm ? sigmoidf_(my_w) * scale : my_w / (tot + 1e-20f) * scale;
   }
 }
 

