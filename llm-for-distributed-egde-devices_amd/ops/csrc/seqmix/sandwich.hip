@@ -33,8 +33,9 @@ __device__ __forceinline__ void group_inv_rms(const float* row_s, float* part_s,
   __syncthreads();
 }
 
-// LDS: row [W] | shares [max(groups, NT / 64)] | inverse rms [groups]
-template <typename T>
+// LDS: row [W] | shares [max(groups, NT / 64)] | inverse rms [groups].  VEC (W % 8 == 0): 8 coordinates per
+// thread and pass, 16- / 32-byte accesses.
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) group_norm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                         T* __restrict__ y, int W, int groups, float eps) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -42,15 +43,34 @@ __global__ void __launch_bounds__(NT) group_norm_kernel(const float* __restrict_
   float* part_s = row_s + W;
   float* inv_s = part_s + max(groups, NT / 64);
   const size_t t = blockIdx.x;
-  for (int c = threadIdx.x; c < W; c += NT) row_s[c] = x[t * W + c];
+  const int gs = W / groups;
+  if constexpr (VEC) {
+    for (int c = threadIdx.x * 8; c < W; c += NT * 8) {
+      float v[8];
+      load8<float>(x + t * W + c, v);
+      store8<float>(row_s + c, v);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += NT) row_s[c] = x[t * W + c];
+  }
   __syncthreads();
   group_inv_rms(row_s, part_s, inv_s, W, groups, eps);
-  const int gs = W / groups;
-  for (int c = threadIdx.x; c < W; c += NT) stf<T>(y + t * W + c, row_s[c] * inv_s[c / gs] * w[c]);
+  if constexpr (VEC) {
+    for (int c = threadIdx.x * 8; c < W; c += NT * 8) {
+      float v[8], wv[8];
+      load8<float>(row_s + c, v);
+      load8<float>(w + c, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] *= inv_s[(c + e) / gs] * wv[e];
+      store8<T>(y + t * W + c, v);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += NT) stf<T>(y + t * W + c, row_s[c] * inv_s[c / gs] * w[c]);
+  }
 }
 
 // x += mult * group-norm(y + sum_k pw[k] parts[k]) w   (y null: the parts alone; pw null: ones)
-template <typename T>
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) group_norm_residual_kernel(float* __restrict__ x, const T* __restrict__ y,
                                                                  const T* __restrict__ parts, const float* __restrict__ pw,
                                                                  int K, const float* __restrict__ w, int W, int groups,
@@ -60,18 +80,49 @@ __global__ void __launch_bounds__(NT) group_norm_residual_kernel(float* __restri
   float* part_s = row_s + W;
   float* inv_s = part_s + max(groups, NT / 64);
   const size_t t = blockIdx.x;
-  for (int c = threadIdx.x; c < W; c += NT) {
-    float v = y ? ldf<T>(y + t * W + c) : 0.f;
-    for (int k = 0; k < K; ++k) {
-      const float p = ldf<T>(parts + (t * K + k) * W + c);
-      v += pw ? pw[t * K + k] * p : p;
+  const int gs = W / groups;
+  if constexpr (VEC) {
+    for (int c = threadIdx.x * 8; c < W; c += NT * 8) {
+      float v[8];
+      if (y) load8<T>(y + t * W + c, v);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = 0.f;
+      }
+      for (int k = 0; k < K; ++k) {
+        float p[8];
+        load8<T>(parts + (t * K + k) * W + c, p);
+        const float pk = pw ? pw[t * K + k] : 1.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += pw ? pk * p[e] : p[e];
+      }
+      store8<float>(row_s + c, v);
     }
-    row_s[c] = v;
+  } else {
+    for (int c = threadIdx.x; c < W; c += NT) {
+      float v = y ? ldf<T>(y + t * W + c) : 0.f;
+      for (int k = 0; k < K; ++k) {
+        const float p = ldf<T>(parts + (t * K + k) * W + c);
+        v += pw ? pw[t * K + k] * p : p;
+      }
+      row_s[c] = v;
+    }
   }
   __syncthreads();
   group_inv_rms(row_s, part_s, inv_s, W, groups, eps);
-  const int gs = W / groups;
-  for (int c = threadIdx.x; c < W; c += NT) x[t * W + c] += mult * (row_s[c] * inv_s[c / gs] * w[c]);
+  if constexpr (VEC) {
+    for (int c = threadIdx.x * 8; c < W; c += NT * 8) {
+      float v[8], wv[8], xv[8];
+      load8<float>(row_s + c, v);
+      load8<float>(w + c, wv);
+      load8<float>(x + t * W + c, xv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[e] += mult * (v[e] * inv_s[(c + e) / gs] * wv[e]);
+      store8<float>(x + t * W + c, xv);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += NT) x[t * W + c] += mult * (row_s[c] * inv_s[c / gs] * w[c]);
+  }
 }
 
 // silu(rw gate) (rw up), rw = the row's router weight (null: 1); u row = gate [ff] | up [ff]
@@ -129,8 +180,12 @@ int edge_sm_group_norm(const float* x, const float* w, void* y, int rows, int W,
   if (rows == 0) return 0;
   if (groups < 1 || W % groups) return -2;
   if (group_norm_lds(W, groups) > 64 * 1024) return -3;
-  SM_T(f32, hipLaunchKernelGGL(group_norm_kernel<T>, dim3(rows), dim3(NT), group_norm_lds(W, groups), st, x, w, (T*)y, W,
-                               groups, eps));
+  if (W % 8 == 0 && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 31) == 0)
+    SM_T(f32, hipLaunchKernelGGL((group_norm_kernel<T, true>), dim3(rows), dim3(NT), group_norm_lds(W, groups), st, x, w,
+                                 (T*)y, W, groups, eps));
+  else
+    SM_T(f32, hipLaunchKernelGGL((group_norm_kernel<T, false>), dim3(rows), dim3(NT), group_norm_lds(W, groups), st, x, w,
+                                 (T*)y, W, groups, eps));
   return (int)hipGetLastError();
 }
 
@@ -139,8 +194,12 @@ int edge_sm_group_norm_residual(float* x, const void* y, const void* parts, cons
   if (rows == 0) return 0;
   if (groups < 1 || W % groups || (!y && K == 0)) return -2;
   if (group_norm_lds(W, groups) > 64 * 1024) return -3;
-  SM_T(f32, hipLaunchKernelGGL(group_norm_residual_kernel<T>, dim3(rows), dim3(NT), group_norm_lds(W, groups), st, x,
-                               (const T*)y, (const T*)parts, pw, K, w, W, groups, eps, mult));
+  if (W % 8 == 0 && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)parts) & 31) == 0)
+    SM_T(f32, hipLaunchKernelGGL((group_norm_residual_kernel<T, true>), dim3(rows), dim3(NT), group_norm_lds(W, groups), st,
+                                 x, (const T*)y, (const T*)parts, pw, K, w, W, groups, eps, mult));
+  else
+    SM_T(f32, hipLaunchKernelGGL((group_norm_residual_kernel<T, false>), dim3(rows), dim3(NT), group_norm_lds(W, groups),
+                                 st, x, (const T*)y, (const T*)parts, pw, K, w, W, groups, eps, mult));
   return (int)hipGetLastError();
 }
 
