@@ -577,6 +577,30 @@ def test_checkpoint_round_trip_and_config(tmp_path):
     assert from_hf_dir(str(out)).layer_specs == model.cfg.layer_specs
 
 
+def test_evaluate_cli_runs_a_checkpoint_folder(tmp_path):
+    """The evaluation command line on a checkpoint folder of this design (vocabulary wide enough for the
+    byte tokenizer): loader by config.json, paged engine and scheduler, the sampling configuration, the
+    confidence metric through the model's own prompt pass."""
+    from edgellm.cli import evaluate
+    cfg = make_config(vocab=300, width=24)
+    d = save(tmp_path, cfg, make_weights(cfg, 3))
+    y = tmp_path / "c.yaml"
+    y.write_text(f"""
+max_new_tokens: 4
+temperature: 0.7
+top_k: 50
+top_p: 0.9
+repetition_penalty: 1.1
+dataset_name: sentence-transformers/natural-questions
+dataset_split: train[:2]
+embedder_model: "none"
+models: ["{d}"]
+""")
+    out = evaluate.main(["--config", str(y), "--devices", "cpu", "--num_samples", "2", "--max_seq", "256",
+                         "--batch_size", "2", "--prefill_chunk", "16", "--precision", "fp32"])
+    assert out[str(d)]["tps"] > 0 and 0 < out[str(d)]["confidence"] <= 1
+
+
 def test_trace_program_on_a_checkpoint_folder(tmp_path):
     """``bin/trace_run`` as a program: steps on standard input, logits files and ``done`` lines out."""
     cfg = CONFIGS["loop_from_0"]()
