@@ -660,6 +660,28 @@ def test_bf16_prompt_attention_on_the_matrix_cores(H, G, D, chunk, cap):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,G,T", [(16, 4, 16400), (12, 6, 11100)])
+def test_prompt_attention_with_grouped_heads_on_long_prompts(H, G, T):
+    """Prompts long enough that the matrix-core kernel serves four (or two) query heads of a kv head from one
+    staged tile: against the general fp32 kernel on the same bf16-rounded inputs (which the oracle pins)."""
+    D, chunk, cap = 32, 700, 25.0
+    g = torch.Generator().manual_seed(1)
+    q = (torch.randn(T, H, D, generator=g) * 0.7).to(torch.bfloat16)
+    k = torch.randn(T, G, D, generator=g).to(torch.bfloat16)
+    gate = torch.randn(T, H * D, generator=g).to(torch.bfloat16)
+    sink, slopes = torch.randn(H, generator=g).cuda(), seqmix.distance_slopes(H, "cuda")
+    outs = []
+    for dt in (torch.float32, torch.bfloat16):
+        cache = _cache("cuda", chunk_attn=_Spec(kv_heads=G, dim=D), pages=(T + 63) // 64, dtype=dt)
+        slot = cache.acquire()
+        meta = _meta(cache, [(slot, 0, T)], "cuda")
+        proj = torch.cat([q.reshape(T, -1), k.reshape(T, -1)], 1).cuda().to(dt)
+        qq = seqmix.rope_paged_write(proj, meta, None, cache.run(0).k, None, H, 0)
+        outs.append(seqmix.chunk_attention(qq, gate.cuda().to(dt), cache.run(0).k, meta, D ** -0.5, chunk, cap, slopes, sink).float().cpu())
+    assert (outs[0] - outs[1]).abs().max() < 0.05
+
+
+@pytest.mark.gpu
 def test_long_chunks_split_over_workgroups_in_decoding():
     """Single-token steps whose chunk holds over a thousand keys: the keys of one query are walked by several
     workgroups and merged; the sink is counted once."""
