@@ -17,6 +17,7 @@ Per run:
       shared key part; a layer that reads another layer's cache holds the same tensor as that run
   canon1 / canon2 [slots, taps - 1, width] fp32                 last inputs of the sublayers' input convolutions
   k = v [pages, page, kv heads, D]                              attention whose values are its keys: one tensor
+  k, v as in the first line for gated attention (the values are cached turned by their position)
 and, for models whose embedding looks at the previous token, ``prev_tok`` int64 [slots].
 A slot's recurrent rows are not cleared on release: a portion that starts at position 0 ignores
 what the slot held (the kernels start from zero there).
@@ -54,6 +55,10 @@ class PagedCache:
                 if chunk_attn is not None:                   # the values are the keys: one row per token serves both
                     rc.k = rc.v = torch.zeros(num_pages, page, chunk_attn.kv_heads, chunk_attn.dim, dtype=dtype,
                                               device=device)
+                elif getattr(s, "gated_attn", None) is not None:
+                    a = s.gated_attn
+                    rc.k = torch.zeros(num_pages, page, a.kv_heads, a.dim, dtype=dtype, device=device)
+                    rc.v = torch.zeros(num_pages, page, a.kv_heads, a.vdim, dtype=dtype, device=device)
                 elif latent is not None:
                     src = s.latent.kv_from
                     if src is None:

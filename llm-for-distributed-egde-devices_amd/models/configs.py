@@ -15,7 +15,9 @@ Families (dims are public HF configs):
                            gated delta-rule layers with mixture-of-experts feed-forwards) and Vetevik
                            (chunked attention with a sink and a distance bias, a gated delta rule
                            with one decay per head, sigmoid-routed experts, norms on both sides of
-                           every sublayer)
+                           every sublayer) and Fikupel (latent attention without positions and gated
+                           grouped-query attention with rotated values, both with a window and a sink,
+                           PolyNorm and mixture-of-experts feed-forwards, several residual streams)
 A single ``ModelConfig`` describes all decoder families; ``DecoderLM`` interprets the flags.
 """
 from __future__ import annotations
@@ -98,6 +100,7 @@ class LatentAttnSpec:
     rot_base: float = 10000.0
     rot_scaling: Optional[dict] = None
     kv_from: Optional[int] = None
+    sink: bool = False           # exp(sink_h), a learned number per head, joins the softmax denominator
 
     @property
     def cache_dim(self) -> int:
@@ -136,6 +139,42 @@ class ChunkAttnSpec:
 
 
 @dataclass
+class GatedAttnSpec:
+    """Grouped-query softmax attention with separate key and value sizes and these parts, each one
+    switchable: an RMS norm per head on q and k before the rotation, one weight vector of ``dim``
+    numbers shared by the heads (``qk_norm``); rotary positions on the first ``rot_dims`` coordinates
+    of each head, neighbouring coordinates (2i, 2i + 1) paired (``rot_scaling``: Llama-3 constants
+    factor / low / high / original); values turned by their own position over all ``vdim``
+    coordinates in the same pairing with frequencies rot_base^(-2m / vdim), cached so, and each
+    head's output turned back by the query's position (``rotate_values``); scores (q . k) scale
+    times a learned number per head (``temp``); a sliding window of ``window`` positions beside the
+    first ``keep_first`` tokens of the sequence, which stay visible at their own positions; exp(sink_h)
+    in the softmax denominator (``sink``); the concatenated heads times sigmoid(W_g h), element by
+    element (``gate``)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: Optional[int] = None
+    keep_first: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[dict] = None   # {"rope_type": "llama3", factor, low_freq_factor, high_freq_factor, original_max_position_embeddings}
+    qk_norm: bool = True
+    rotate_values: bool = True
+    temp: bool = True
+    sink: bool = True
+    gate: bool = True
+
+    @property
+    def proj_sizes(self):
+        """Row blocks of the fused input projection: q | k | v | gate."""
+        return (self.heads * self.dim, self.kv_heads * self.dim, self.kv_heads * self.vdim,
+                self.heads * self.vdim if self.gate else 0)
+
+
+@dataclass
 class DeltaSpec:
     """Gated delta rule: a [dim, vdim] fp32 state per head, q / k shared by ``heads / kv_heads`` heads,
     a causal depthwise convolution of ``conv`` taps + silu over q | k | v, unit-length q and k, an RMS
@@ -171,7 +210,8 @@ class DeltaSpec:
 class MoESpec:
     """Mixture of gated-linear experts.  ``router`` "softmax": softmax over ``experts``, the ``top``
     largest renormalised and multiplied by ``scale``; "sigmoid": scores sigmoid(W_r h), the ``top``
-    largest taken as they are.  ``act`` "glu_clamp": g = min(W_g h, limit), u = clamp(W_u h, +-limit),
+    largest taken as they are; "top_softmax": the ``top`` largest logits (W_r h + b with ``router_bias``),
+    softmax over the chosen ones only.  ``act`` "glu_clamp": g = min(W_g h, limit), u = clamp(W_u h, +-limit),
     W_d (g sigmoid(1.702 g) (u + 1)); "silu_glu": W_d (silu(W_g h) (W_u h)).  ``weight_on`` "output":
     the result is sum_k w_k expert_k(h); "input": sum_k expert_k(w_k h).  An optional shared expert of
     width ``shared_ff`` runs for every token."""
@@ -185,6 +225,7 @@ class MoESpec:
     router: str = "softmax"
     act: str = "glu_clamp"
     weight_on: str = "output"
+    router_bias: bool = False
 
 
 @dataclass
@@ -194,14 +235,17 @@ class LayerSpec:
     mixer: str                               # "parallel": attention and state-space side by side;
                                              # "latent_attention" / "channel_delta": one mixer, norm on the sublayer's output;
                                              # "chunk_attention" / "head_delta": one mixer, norms on both sides of each sublayer
+                                             # "gated_attention" (and "latent_attention" in a model with ``streams``):
+                                             # one mixer, a norm before each sublayer, several residual streams
     attn: Optional[WindowAttnSpec] = None
     ssd: Optional[SSDSpec] = None
     ff: Optional[int] = None
-    ff_act: str = "relu2"
+    ff_act: str = "relu2"                    # "relu2" | "polynorm" (a N(z) + b N(z^2) + c N(z^3) + e, N = divide by the row's rms)
     latent: Optional[LatentAttnSpec] = None
     delta: Optional[DeltaSpec] = None
     moe: Optional[MoESpec] = None
     chunk_attn: Optional[ChunkAttnSpec] = None
+    gated_attn: Optional[GatedAttnSpec] = None
 
 
 @dataclass
@@ -257,6 +301,11 @@ class ModelConfig:
     # is multiplied by ``residual_mult`` before it joins the stream
     norm_groups: int = 1
     residual_mult: float = 1.0
+    # arch "fikupel": pre-norm layers over ``streams`` copies of the residual stream (hyper-connections:
+    # a sublayer reads a weighted sum of the streams, and every stream becomes a mix of all of them plus its
+    # own multiple of the sublayer's output); ``hyper`` False: one stream with the plain residual sum
+    streams: int = 0
+    hyper: bool = True
 
     def layer_runs(self) -> List[tuple]:
         """[(layer index, pass number or None)] in execution order; every run has its own cache."""
@@ -441,7 +490,7 @@ def checkpoint_shapes(path: str) -> dict:
 def from_hf_dir(path: str) -> ModelConfig:
     with open(os.path.join(path, "config.json")) as f:
         c = json.load(f)
-    needs_shapes = str(c.get("architecture", "")).lower() == "pagonex"
+    needs_shapes = str(c.get("architecture", "")).lower() in ("pagonex", "fikupel")
     return from_hf_config(c, checkpoint_shapes(path) if needs_shapes else None)
 
 
@@ -677,6 +726,102 @@ def to_vetevik_config(cfg: ModelConfig) -> dict:
     return out
 
 
+def _llama3_scaling(sc: Optional[dict]) -> Optional[dict]:
+    """{factor, low, high, original} -> the ``rope_tables`` form of the Llama-3 frequency rule."""
+    if not sc:
+        return None
+    return {"rope_type": "llama3", "factor": float(sc["factor"]), "low_freq_factor": float(sc["low"]),
+            "high_freq_factor": float(sc["high"]), "original_max_position_embeddings": float(sc["original"])}
+
+
+def from_fikupel_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
+    """The Fikupel layout of ``config.json``: ``layers`` (``type`` = ``latent_attention`` or ``attention``,
+    ``mixer`` sizes and constants, ``mlp`` = dense, mixture of experts or null), ``streams``, ``norm.eps``,
+    ``vocab``, ``width``.  The embedding table is also the output projection.  What a mixer's entry leaves
+    out does not exist (no ``mask``: every earlier token is seen; no ``rot``: nothing is rotated).
+    ``shapes`` (tensor name -> shape of the checkpoint) tells whether the optional per-head tensors and the
+    stream weights are there."""
+    has = (lambda name: name in shapes) if shapes is not None else (lambda name: True)
+    specs = []
+    for i, l in enumerate(c["layers"]):
+        m, kind = l["mixer"], l["type"]
+        mask = m.get("mask") or {}
+        window = int(mask["size"]) if mask.get("size") is not None else None
+        lat = ga = None
+        if kind == "latent_attention":
+            lat = LatentAttnSpec(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=0, vdim=int(m["vdim"]),
+                                 q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
+                                 window=window, sink=has(f"l{i}.mix.sink"))
+        elif kind == "attention":
+            rot = m.get("rot") or None
+            ga = GatedAttnSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
+                               vdim=int(m["vdim"]), scale=float(m["scale"]), window=window,
+                               keep_first=int(mask.get("keep_first", 0) or 0) if window is not None else 0,
+                               rot_dims=int(rot["dims"]) if rot else 0, rot_base=float(rot["base"]) if rot else 10000.0,
+                               rot_scaling=_llama3_scaling(rot.get("scaling")) if rot else None,
+                               qk_norm=has(f"l{i}.mix.q.norm"), rotate_values=bool(rot), temp=has(f"l{i}.mix.temp"),
+                               sink=has(f"l{i}.mix.sink"), gate=has(f"l{i}.mix.g"))
+            if ga.heads % ga.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+            if ga.rot_dims % 2 or ga.rot_dims > ga.dim or (ga.rotate_values and ga.vdim % 2):
+                raise ValueError("rotation runs over pairs of coordinates inside a head")
+        else:
+            raise ValueError(f"unsupported layer type {kind!r}")
+        mlp, moe, ff = l.get("mlp") or None, None, None
+        if mlp and mlp.get("kind", "dense") == "dense":
+            ff = int(mlp["ff"])
+        elif mlp and mlp.get("kind") == "moe":
+            r = mlp["router"]
+            moe = MoESpec(experts=int(r["experts"]), top=int(r["top"]), scale=1.0, ff=int(mlp["expert"]["ff"]),
+                          router="top_softmax", act="silu_glu", weight_on="output", router_bias=has(f"l{i}.mlp.router.b"))
+        elif mlp:
+            raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}")
+        specs.append(LayerSpec("latent_attention" if lat else "gated_attention", ff=ff, ff_act="polynorm", latent=lat,
+                               moe=moe, gated_attn=ga))
+    first = specs[0].latent or specs[0].gated_attn
+    return ModelConfig(arch="fikupel", vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), num_layers=len(specs),
+                       num_heads=first.heads, num_kv_heads=getattr(first, "kv_heads", 1), intermediate_size=0,
+                       head_dim=first.dim, max_position_embeddings=1 << 20, norm="rms", norm_eps=float(c["norm"]["eps"]),
+                       act="silu_glu", pos_emb="rope", tie_word_embeddings=True, name=c.get("name", "fikupel"),
+                       layer_specs=specs, streams=int(c.get("streams") or 1),
+                       hyper=("streams" in c and c["streams"] is not None) and has("l0.hc1.in"))
+
+
+def to_fikupel_config(cfg: ModelConfig) -> dict:
+    """Inverse of ``from_fikupel_config``."""
+    layers = []
+    for s in cfg.layer_specs:
+        if s.latent is not None:
+            a = s.latent
+            m = {"heads": a.heads, "dim": a.dim, "vdim": a.vdim, "q_rank": a.q_rank, "kv_rank": a.kv_rank, "scale": a.scale}
+            if a.window is not None:
+                m["mask"] = {"size": a.window}
+            kind = "latent_attention"
+        else:
+            a = s.gated_attn
+            m = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale}
+            if a.window is not None:
+                m["mask"] = {"size": a.window, "keep_first": a.keep_first}
+            if a.rot_dims or a.rotate_values:
+                m["rot"] = {"dims": a.rot_dims, "base": a.rot_base}
+                if a.rot_scaling:
+                    r = a.rot_scaling
+                    m["rot"]["scaling"] = {"factor": r["factor"], "low": r["low_freq_factor"], "high": r["high_freq_factor"],
+                                           "original": r["original_max_position_embeddings"]}
+            kind = "attention"
+        mlp = None
+        if s.moe is not None:
+            mlp = {"kind": "moe", "router": {"experts": s.moe.experts, "top": s.moe.top}, "expert": {"ff": s.moe.ff}}
+        elif s.ff:
+            mlp = {"kind": "dense", "ff": s.ff}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    out = {"architecture": "Fikupel", "vocab": cfg.vocab_size, "width": cfg.hidden_size, "layers": layers,
+           "norm": {"eps": cfg.norm_eps}}
+    if cfg.hyper:
+        out["streams"] = cfg.streams
+    return out
+
+
 def from_hf_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
     """Map a ``config.json`` onto ModelConfig (Hugging Face ``model_type`` layouts, or an
     ``architecture`` key naming a per-layer layout; ``shapes``: the checkpoint's tensor shapes, for
@@ -687,6 +832,8 @@ def from_hf_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
         return from_pagonex_config(c, shapes)
     if str(c.get("architecture", "")).lower() == "vetevik":
         return from_vetevik_config(c)
+    if str(c.get("architecture", "")).lower() == "fikupel":
+        return from_fikupel_config(c, shapes)
     mt = c.get("model_type")
     eos = c.get("eos_token_id")
     if isinstance(eos, list):

@@ -250,10 +250,11 @@ def save_hf_model(model: DecoderLM, path: str, shard_bytes: int = 4 << 30) -> st
     """Write ``config.json`` + safetensors shards readable by both edgellm and transformers
     (layer-spec models: their own config layout and tensor names)."""
     from safetensors.torch import save_file
-    from .configs import to_hf_config, to_nudadra_config, to_pagonex_config, to_vetevik_config
+    from .configs import to_fikupel_config, to_hf_config, to_nudadra_config, to_pagonex_config, to_vetevik_config
     os.makedirs(path, exist_ok=True)
     spec_model = model.cfg.layer_specs is not None
-    to_spec = {"pagonex": to_pagonex_config, "vetevik": to_vetevik_config}.get(model.cfg.arch, to_nudadra_config)
+    to_spec = {"pagonex": to_pagonex_config, "vetevik": to_vetevik_config,
+               "fikupel": to_fikupel_config}.get(model.cfg.arch, to_nudadra_config)
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(to_spec(model.cfg) if spec_model else to_hf_config(model.cfg), f, indent=2)
     if spec_model:

@@ -1,4 +1,4 @@
-"""Layer-spec language models (arch "nudadra", "pagonex", "vetevik"): every layer is described by its own
+"""Layer-spec language models (arch "nudadra", "pagonex", "vetevik", "fikupel"): every layer is described by its own
 entry of ``ModelConfig.layer_specs``, a span of layers may run several times in a row, and the
 residual stream is fp32.
 
@@ -13,6 +13,14 @@ x <- x + m N2b(ff(N2(x))), every N an RMS norm in groups with its own weight vec
 for the model.  The mixer is chunked attention with a sink or a gated delta rule with a decay per
 head, the feed-forward a sigmoid-routed mixture of experts; a looped span adds the embedding rows
 to the stream before every pass but the first; the embedding table is the output projection.
+
+Per layer (norm before each sublayer over several streams, ``HyperLayer``): the residual stream exists
+in S copies x_1 .. x_S (all equal to the embedding rows at the start).  A sublayer reads
+u = sum_s a_s x_s, computes y = f(RMSnorm(u)), and every stream becomes x_r <- sum_s M[s, r] x_s + b_r y
+(a, M, b learned per sublayer); with one stream and no such weights this is x <- x + f(norm(x)).  The
+mixer is latent attention without positions or gated grouped-query attention, the feed-forward a
+PolyNorm unit or a mixture of experts; the final norm reads the sum of the streams and the embedding
+table is the output projection.
 
 Per layer (parallel form):  h = norm(x) ;  x <- x + mixer(h) + ff(h), with one norm whose gain is a
 single number, a ``ParallelMixer`` (models/mixers.py) and a squared-ReLU feed-forward.  The
@@ -38,7 +46,8 @@ import torch.nn as nn
 from ..ops import seqmix
 from .configs import LayerSpec, ModelConfig
 from .layers import GroupRMSNorm, Linear, RowLayerNorm, ScalarNorm
-from .mixers import ChannelDeltaMixer, ChunkAttention, HeadDeltaMixer, LatentAttention, ParallelMixer
+from .mixers import (ChannelDeltaMixer, ChunkAttention, GatedAttention, HeadDeltaMixer, LatentAttention,
+                     ParallelMixer)
 from .moe import MoEFeedForward
 
 
@@ -125,7 +134,93 @@ class SandwichLayer(nn.Module):
         return x
 
 
+class StreamNorm(nn.Module):
+    """RMS norm with a weight vector over a weighted sum of the residual streams [T, S, W] (fp32):
+    ``in_w`` fp32 [S] or None for the plain sum (one stream: the stream itself)."""
+
+    def __init__(self, width: int, eps: float, device=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, X: torch.Tensor, in_w: Optional[torch.Tensor], out_dtype=torch.bfloat16) -> torch.Tensor:
+        return seqmix.hyper_read_norm(X, in_w, self.weight, self.eps, out_dtype)
+
+
+class HyperConnection(nn.Module):
+    """The weights that tie one sublayer to S residual streams: ``inp`` [S] (what the sublayer reads),
+    ``mix`` [S, S] indexed [from, to] and ``out`` [S] (how every stream is rebuilt from all of them and
+    the sublayer's output)."""
+
+    def __init__(self, streams: int, device=None):
+        super().__init__()
+        P = lambda t: nn.Parameter(t.to(device), requires_grad=False)
+        self.inp = P(torch.full((streams,), 1.0 / streams, dtype=torch.float32))
+        self.mix = P(torch.eye(streams, dtype=torch.float32))
+        self.out = P(torch.ones(streams, dtype=torch.float32))
+
+
+class PolyNormFF(nn.Module):
+    """W_down act(W_up h) with act(z) = a N(z) + b N(z^2) + c N(z^3) + e over each token's ff values."""
+
+    def __init__(self, width: int, ff: int, eps: float, dtype, device):
+        super().__init__()
+        self.eps = eps
+        self.up = Linear(width, ff, False, dtype, device)
+        self.down = Linear(ff, width, False, dtype, device)
+        self.act = nn.Parameter(torch.zeros(4, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return self.down(seqmix.poly_norm(self.up(h), self.act, self.eps))
+
+
+class HyperLayer(nn.Module):
+    """One mixer (latent attention without positions or gated attention) and an optional feed-forward
+    (PolyNorm unit or mixture of experts), each reading the RMS norm of a weighted sum of the residual
+    streams and written back into all of them; one stream without weights: the plain pre-norm residual."""
+
+    def __init__(self, cfg: ModelConfig, spec: LayerSpec, idx: int, dtype, device):
+        super().__init__()
+        W, eps = cfg.hidden_size, cfg.norm_eps
+        self.idx, self.spec, self.dtype = idx, spec, dtype
+        if spec.mixer == "latent_attention":
+            self.mix = LatentAttention(spec.latent, W, eps, dtype, device)
+        elif spec.mixer == "gated_attention":
+            self.mix = GatedAttention(spec.gated_attn, W, eps, dtype, device)
+        else:
+            raise ValueError(spec.mixer)
+        self.norm1 = StreamNorm(W, eps, device)
+        self.hc1 = HyperConnection(cfg.streams, device) if cfg.hyper else None
+        if spec.moe is not None:
+            self.ff = MoEFeedForward(spec.moe, W, dtype, device)
+        elif spec.ff:
+            assert spec.ff_act == "polynorm", spec.ff_act
+            self.ff = PolyNormFF(W, spec.ff, eps, dtype, device)
+        else:
+            self.ff = None
+        if self.ff is not None:
+            self.norm2 = StreamNorm(W, eps, device)
+            self.hc2 = HyperConnection(cfg.streams, device) if cfg.hyper else None
+
+    def forward(self, X: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        hc = self.hc1
+        y = self.mix(self.norm1(X, hc.inp if hc is not None else None, self.dtype), meta, run)
+        seqmix.hyper_update(X, hc.mix if hc is not None else None, hc.out if hc is not None else None, y)
+        if self.ff is not None:
+            hc = self.hc2
+            h = self.norm2(X, hc.inp if hc is not None else None, self.dtype)
+            mix, out = (hc.mix, hc.out) if hc is not None else (None, None)
+            if self.spec.moe is not None:
+                shared, parts, wts = self.ff(h)
+                seqmix.hyper_update(X, mix, out, shared, parts, wts)
+            else:
+                seqmix.hyper_update(X, mix, out, self.ff(h))
+        return X
+
+
 def _make_layer(cfg: ModelConfig, spec: LayerSpec, idx: int, dtype, device) -> nn.Module:
+    if cfg.streams:
+        return HyperLayer(cfg, spec, idx, dtype, device)
     if spec.mixer == "parallel":
         return HybridLayer(cfg, spec, idx, dtype, device)
     if spec.mixer in ("chunk_attention", "head_delta"):
@@ -153,7 +248,8 @@ class HybridLM(nn.Module):
             self.loop_in = Linear(2 * W, W, False, dtype, device)
             self.loop_step = nn.Parameter(torch.zeros(cfg.loop.times, W, dtype=torch.float32, device=device),
                                           requires_grad=False)
-        self.final_norm = ScalarNorm(cfg.norm_eps, device) if cfg.norm == "rms_scalar" else \
+        self.final_norm = StreamNorm(W, cfg.norm_eps, device) if cfg.streams else \
+            ScalarNorm(cfg.norm_eps, device) if cfg.norm == "rms_scalar" else \
             GroupRMSNorm(W, cfg.norm_groups, cfg.norm_eps, device) if cfg.norm == "rms_group" else \
             RowLayerNorm(W, cfg.norm_eps, device)
         self.lm_head = Linear(W, cfg.vocab_size, False, dtype, device)
@@ -190,6 +286,8 @@ class HybridLM(nn.Module):
         else:
             x0 = seqmix.embedding_scaled(ids, self.embed, cfg.embed_scale)
         x = x0.clone() if cfg.loop is not None else x0
+        if cfg.streams:                                  # [T, S, W]: every stream starts as the embedding rows
+            x = x0[:, None, :].expand(-1, cfg.streams, -1).contiguous()
         for r, (i, t) in enumerate(self.runs):
             if t is not None and i == cfg.loop.start:
                 if cfg.loop.entry == "add_embed":
@@ -199,12 +297,12 @@ class HybridLM(nn.Module):
                     x = seqmix.linear_f32(seqmix.cat_cast(x, x0, self.dtype), self.loop_in.weight, self.loop_step[t])
             x = self.layers[i](x, meta, cache.run(r))
             if taps is not None:
-                taps.append(x.clone())
+                taps.append(x.sum(1) if cfg.streams else x.clone())
         if rows is not None:
             if rows.numel() == 0:                        # nothing asked for: the step only fed the cache
                 return torch.empty(0, cfg.vocab_size, dtype=torch.float32, device=x.device)
             x = x.index_select(0, rows)
-        h = self.final_norm(x, self.dtype)
+        h = self.final_norm(x, None, self.dtype) if cfg.streams else self.final_norm(x, self.dtype)
         logits = self.lm_head(h).float()
         return logits if cfg.logit_scale == 1.0 else logits.mul_(cfg.logit_scale)
 
@@ -418,9 +516,102 @@ def export_vetevik_tensors(model: "HybridLM") -> Dict[str, torch.Tensor]:
     return {k: v.to(torch.bfloat16).contiguous() for k, v in out.items()}
 
 
+def convert_fikupel_tensors(cfg: ModelConfig, t: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    """Checkpoint names of the Fikupel layout (``l<i>.mix.dq``, ``l<i>.hc1.mix``, ``l<i>.mlp.e<k>.gate`` ...) ->
+    this package's parameter names: fused input projections, per-head key / value expansions, stacked
+    expert weights."""
+    out = {"embed": t["embed"], "final_norm.weight": t["final.norm"]}
+    for i, spec in enumerate(cfg.layer_specs):
+        p, o = f"l{i}.", f"layers.{i}."
+        M, m = p + "mix.", o + "mix."
+        has_ff = spec.moe is not None or bool(spec.ff)
+        for n in ("1", "2") if has_ff else ("1",):
+            out[o + f"norm{n}.weight"] = t[p + f"norm{n}"]
+            if cfg.hyper:
+                for ours, theirs in (("inp", "in"), ("mix", "mix"), ("out", "out")):
+                    out[o + f"hc{n}.{ours}"] = t[p + f"hc{n}.{theirs}"]
+        if spec.latent is not None:
+            a = spec.latent
+            out[m + "proj_in.weight"] = torch.cat([t[M + "dq"], t[M + "dkv"]], 0)
+            out[m + "q_norm"], out[m + "kv_norm"] = t[M + "dq.norm"], t[M + "dkv.norm"]
+            out[m + "uq.weight"] = t[M + "uq"]
+            out[m + "uk"] = t[M + "uk"].reshape(a.heads, a.dim, a.kv_rank)
+            out[m + "uv"] = t[M + "uv"].reshape(a.heads, a.vdim, a.kv_rank).transpose(1, 2).contiguous()
+        else:
+            a = spec.gated_attn
+            out[m + "proj_in.weight"] = torch.cat([t[M + n] for n in ("q", "k", "v") + (("g",) if a.gate else ())], 0)
+            if a.qk_norm:
+                out[m + "q_norm"], out[m + "k_norm"] = t[M + "q.norm"], t[M + "k.norm"]
+            if a.temp:
+                out[m + "temp"] = t[M + "temp"]
+        if a.sink:
+            out[m + "sink"] = t[M + "sink"]
+        out[m + "o.weight"] = t[M + "o"]
+        F_, f = p + "mlp.", o + "ff."
+        if spec.moe is not None:
+            e = spec.moe
+            out[f + "router"] = t[F_ + "router"]
+            if e.router_bias:
+                out[f + "router_b"] = t[F_ + "router.b"]
+            out[f + "w_gu"] = torch.stack([torch.cat([t[f"{F_}e{k}.gate"], t[f"{F_}e{k}.up"]], 0) for k in range(e.experts)])
+            out[f + "w_down"] = torch.stack([t[f"{F_}e{k}.down"] for k in range(e.experts)])
+        elif spec.ff:
+            out[f + "up.weight"], out[f + "down.weight"], out[f + "act"] = t[F_ + "up"], t[F_ + "down"], t[F_ + "act"]
+    return out
+
+
+def export_fikupel_tensors(model: "HybridLM") -> Dict[str, torch.Tensor]:
+    """Inverse of ``convert_fikupel_tensors`` (checkpoint names, 16-bit storage)."""
+    cfg = model.cfg
+    p = {k: v.detach() for k, v in model.named_parameters()}
+    out = {"embed": p["embed"], "final.norm": p["final_norm.weight"]}
+    for i, spec in enumerate(cfg.layer_specs):
+        q, o = f"l{i}.", f"layers.{i}."
+        M, m = q + "mix.", o + "mix."
+        has_ff = spec.moe is not None or bool(spec.ff)
+        for n in ("1", "2") if has_ff else ("1",):
+            out[q + f"norm{n}"] = p[o + f"norm{n}.weight"]
+            if cfg.hyper:
+                for ours, theirs in (("inp", "in"), ("mix", "mix"), ("out", "out")):
+                    out[q + f"hc{n}.{theirs}"] = p[o + f"hc{n}.{ours}"]
+        w = p[m + "proj_in.weight"]
+        if spec.latent is not None:
+            a = spec.latent
+            out[M + "dq"], out[M + "dkv"] = w[:a.q_rank], w[a.q_rank:]
+            out[M + "dq.norm"], out[M + "dkv.norm"] = p[m + "q_norm"], p[m + "kv_norm"]
+            out[M + "uq"] = p[m + "uq.weight"]
+            out[M + "uk"] = p[m + "uk"].reshape(a.heads * a.dim, a.kv_rank)
+            out[M + "uv"] = p[m + "uv"].transpose(1, 2).reshape(a.heads * a.vdim, a.kv_rank)
+        else:
+            a = spec.gated_attn
+            for n, part in zip(("q", "k", "v", "g"), torch.split(w, list(a.proj_sizes), 0)):
+                if part.shape[0]:
+                    out[M + n] = part
+            if a.qk_norm:
+                out[M + "q.norm"], out[M + "k.norm"] = p[m + "q_norm"], p[m + "k_norm"]
+            if a.temp:
+                out[M + "temp"] = p[m + "temp"]
+        if a.sink:
+            out[M + "sink"] = p[m + "sink"]
+        out[M + "o"] = p[m + "o.weight"]
+        F_, f = q + "mlp.", o + "ff."
+        if spec.moe is not None:
+            e = spec.moe
+            out[F_ + "router"] = p[f + "router"]
+            if e.router_bias:
+                out[F_ + "router.b"] = p[f + "router_b"]
+            for k in range(e.experts):
+                out[f"{F_}e{k}.gate"], out[f"{F_}e{k}.up"] = p[f + "w_gu"][k, :e.ff], p[f + "w_gu"][k, e.ff:]
+                out[f"{F_}e{k}.down"] = p[f + "w_down"][k]
+        elif spec.ff:
+            out[F_ + "up"], out[F_ + "down"], out[F_ + "act"] = p[f + "up.weight"], p[f + "down.weight"], p[f + "act"]
+    return {k: v.to(torch.bfloat16).contiguous() for k, v in out.items()}
+
+
 CONVERTERS = {"nudadra": (convert_nudadra_tensors, export_nudadra_tensors),
               "pagonex": (convert_pagonex_tensors, export_pagonex_tensors),
-              "vetevik": (convert_vetevik_tensors, export_vetevik_tensors)}
+              "vetevik": (convert_vetevik_tensors, export_vetevik_tensors),
+              "fikupel": (convert_fikupel_tensors, export_fikupel_tensors)}
 
 
 @torch.no_grad()
@@ -464,8 +655,20 @@ def init_random_hybrid_(model: HybridLM, seed: int = 0) -> HybridLM:
             v = r(*p.shape) / p.shape[-1 if leaf in ("w_gu", "w_down") else 1] ** 0.5
         elif leaf == "router" or name == "bigram":
             v = r(*p.shape) * (0.5 if name == "bigram" else 1.0)
-        elif leaf in ("q_norm", "kv_norm"):
+        elif leaf in ("q_norm", "kv_norm", "k_norm"):
             v = 1.0 + 0.1 * r(*p.shape)
+        elif leaf == "temp":
+            v = 1.0 + 0.2 * torch.rand(*p.shape, generator=g)
+        elif leaf == "inp":                              # stream weights: near an even read, a near-identity mix, outputs near 1
+            v = 1.0 / p.shape[0] + 0.1 * r(*p.shape)
+        elif leaf == "mix" and p.dim() == 2:
+            v = torch.eye(p.shape[0]) + 0.1 * r(*p.shape)
+        elif leaf == "out" and p.dim() == 1:
+            v = 1.0 + 0.1 * r(*p.shape)
+        elif leaf == "act":
+            v = torch.tensor([1.0, 0.5, 0.25, 0.0]) + 0.1 * r(*p.shape)
+        elif leaf == "router_b":
+            v = 0.5 * r(*p.shape)
         elif leaf == "sink":
             v = r(*p.shape)
         elif leaf in ("canon1", "canon2"):

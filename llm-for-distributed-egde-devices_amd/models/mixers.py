@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 
 from ..ops import seqmix
-from .configs import ChunkAttnSpec, DeltaSpec, SSDSpec, WindowAttnSpec
+from .configs import ChunkAttnSpec, DeltaSpec, GatedAttnSpec, SSDSpec, WindowAttnSpec
 from .layers import Linear
 
 
@@ -152,7 +152,8 @@ class LatentAttention(nn.Module):
     attention runs as one kv head of size kv_rank + R over the cached rows themselves, with the
     latent as the value; each head's weighted latent is then expanded by W_uv,h.  The cache is read
     once for all heads and nothing per head is stored.  A layer with ``kv_from`` reads another
-    layer's cached rows and has no down projection of its own."""
+    layer's cached rows and has no down projection of its own.  ``rot_dim`` 0: no rotated part at all
+    (attention without positions); ``sink``: a learned number per head in the softmax denominator."""
 
     def __init__(self, spec, width: int, eps: float, dtype, device):
         super().__init__()
@@ -168,6 +169,7 @@ class LatentAttention(nn.Module):
         self.uk = nn.Parameter(torch.zeros(s.heads, s.dim, s.kv_rank, dtype=dtype, device=device), requires_grad=False)
         self.uv = nn.Parameter(torch.zeros(s.heads, s.kv_rank, s.vdim, dtype=dtype, device=device), requires_grad=False)
         self.o = Linear(s.heads * s.vdim, width, False, dtype, device)
+        self.sink = P(s.heads) if s.sink else None
         self._rope = {}
 
     def forward(self, h: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
@@ -181,9 +183,44 @@ class LatentAttention(nn.Module):
         qc = seqmix.latent_write(u if self.own_kv else None, s.q_rank, self.kv_norm, self.eps, q, q_lat, meta, rope,
                                  run.lat, s.kv_rank, s.rot_dims)
         a = seqmix.window_pool_attention(qc, None, run.lat, run.lat[..., :s.kv_rank], None, None, meta, s.scale,
-                                         s.window, None)                                # [T, H * kv_rank]
+                                         s.window, None, self.sink)                     # [T, H * kv_rank]
         v = torch.bmm(a.view(T, H, s.kv_rank).transpose(0, 1), self.uv).transpose(0, 1)  # [T, H, vdim]
         return self.o(v.reshape(T, H * s.vdim))
+
+
+class GatedAttention(nn.Module):
+    """Grouped-query attention with an RMS norm per head on q and k, rotary positions on part of each
+    head (neighbouring coordinates paired), values cached turned by their own position and each head's
+    output turned back by the query's, a learned temperature and a learned sink per head, a sliding
+    window beside the sequence's first tokens, and an element-wise sigmoid gate from the same input.
+    One fused GEMM produces q | k | v | gate; the temperature is folded into q in fp32."""
+
+    def __init__(self, spec: GatedAttnSpec, width: int, eps: float, dtype, device):
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        s = spec
+        P = lambda *shape: nn.Parameter(torch.zeros(*shape, dtype=torch.float32, device=device), requires_grad=False)
+        self.proj_in = Linear(width, sum(s.proj_sizes), False, dtype, device)
+        self.q_norm = P(s.dim) if s.qk_norm else None
+        self.k_norm = P(s.dim) if s.qk_norm else None
+        self.temp = P(s.heads) if s.temp else None
+        self.sink = P(s.heads) if s.sink else None
+        self.o = Linear(s.heads * s.vdim, width, False, dtype, device)
+        self._rope, self._vrope = {}, {}
+
+    def forward(self, h: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        s = self.spec
+        nq, nk, nv, ng = s.proj_sizes
+        u = self.proj_in(h)
+        rope = _shared_rope(self._rope, (s.rot_dims, s.rot_base, s.rot_scaling), meta.max_keys, h.device)
+        vrope = _shared_rope(self._vrope, (s.vdim, s.rot_base, None), meta.max_keys, h.device) if s.rotate_values else None
+        q = seqmix.qk_norm_rope_write(u, meta, self.q_norm, self.k_norm, self.eps, rope, vrope, self.temp, run.k, run.v,
+                                      s.heads, s.rot_dims)
+        a = seqmix.window_pool_attention(q, None, run.k, run.v, None, None, meta, s.scale, s.window, None, self.sink,
+                                         s.keep_first)
+        if vrope is not None or ng:
+            a = seqmix.unrotate_gate(a, u[:, nq + nk + nv:nq + nk + nv + ng] if ng else None, meta, vrope, s.heads)
+        return self.o(a)
 
 
 class ChannelDeltaMixer(nn.Module):

@@ -1,7 +1,8 @@
 """Mixture-of-experts feed-forward for layer-spec models.
 
 Router: softmax over all experts in fp32, the ``top`` largest scores renormalised and scaled, or
-sigmoid scores taken as they are (``ops.seqmix.moe_route``).  Experts: clamped or plain silu
+sigmoid scores taken as they are, or the ``top`` largest logits (with a bias) and a softmax over those
+alone (``ops.seqmix.moe_route``).  Experts: clamped or plain silu
 gated-linear units, the router's weight on their output or on their input, weights stacked per layer as
 ``w_gu`` [E, 2 ff, W] (gate rows, then up rows) and ``w_down`` [E, W, ff]; decode-sized steps read
 only the chosen experts' rows, prompt-sized steps sort (token, choice) pairs by expert
@@ -25,6 +26,8 @@ class MoEFeedForward(nn.Module):
         self.spec = spec
         s = spec
         self.router = nn.Parameter(torch.zeros(s.experts, width, dtype=torch.float32, device=device), requires_grad=False)
+        self.router_b = nn.Parameter(torch.zeros(s.experts, dtype=torch.float32, device=device), requires_grad=False) \
+            if s.router_bias else None
         self.w_gu = nn.Parameter(torch.zeros(s.experts, 2 * s.ff, width, dtype=dtype, device=device), requires_grad=False)
         self.w_down = nn.Parameter(torch.zeros(s.experts, width, s.ff, dtype=dtype, device=device), requires_grad=False)
         if s.shared_ff:
@@ -35,7 +38,7 @@ class MoEFeedForward(nn.Module):
         """h [T, W] -> (shared expert's output [T, W] or None, expert outputs [T, top, W], weights fp32
         [T, top] still to be applied to them, or None when the experts ran on weighted inputs)."""
         s = self.spec
-        idx, wts = seqmix.moe_route(h, self.router, s.top, s.scale, s.router)
+        idx, wts = seqmix.moe_route(h, self.router, s.top, s.scale, s.router, self.router_b)
         on_input = s.weight_on == "input"
         parts = seqmix.moe_experts(h, idx, self.w_gu, self.w_down, s.limit, s.act, wts if on_input else None)
         if on_input:

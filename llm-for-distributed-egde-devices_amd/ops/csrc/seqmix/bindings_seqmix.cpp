@@ -35,14 +35,14 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
                       int window, int pool, int f32, int nsplit, float* part, int kld, int vld, int chunked, float cap,
-                      const float* slopes, const float* sink, int gate_elem, hipStream_t st);
+                      const float* slopes, const float* sink, int gate_elem, int keep_first, hipStream_t st);
 size_t edge_sm_attention_part_floats(int rows, int H, int G, int D, int Dv, int nsplit);
 int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp,
                            const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
                            const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
                            int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
                            int pool, int kld, int vld, int chunked, float cap, const float* slopes, const float* sink,
-                           int gate_elem, hipStream_t st);
+                           int gate_elem, int keep_first, hipStream_t st);
 int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
                       const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
                       const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
@@ -79,8 +79,20 @@ int edge_sm_delta_prep(const void* qkv, int Cq, const void* u, int ld, int b0, c
 int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, float* state, const int* seq_slot,
                        const int* seq_start, const int* seq_len, const int* seq_off, float* y, int n, int H, int G, int N,
                        int P, int GD, int f32, hipStream_t st);
-int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, float* z, int* idx, float* wts,
-                      int rows, int sigm, int f32, hipStream_t st);
+int edge_sm_moe_route(const void* h, int W, const float* router, const float* bias, int E, int top, float scale, float* z,
+                      int* idx, float* wts, int rows, int sigm, int f32, hipStream_t st);
+int edge_sm_hyper_read_norm(const float* X, const float* in_w, const float* w, void* y, int rows, int S, int W, float eps,
+                            int f32, hipStream_t st);
+int edge_sm_hyper_update(float* X, const float* mix, const float* out_w, const void* y, const void* parts, const float* pw,
+                         int K, int rows, int S, int W, int f32, hipStream_t st);
+int edge_sm_poly_norm(const void* z, int ld, const float* coef, void* y, int rows, int F, float eps, int f32,
+                      hipStream_t st);
+int edge_sm_qk_norm_rope_write(const void* proj, int ld, const int* tok_seq, const int* tok_pos, const int* seq_slot,
+                               const int* ptab, int ptab_ld, const float* qw, const float* kw, float eps, const float* cs,
+                               const float* vcs, const float* temp, void* q_out, void* kp, void* vp, int rows, int H, int G,
+                               int D, int Dv, int rot, int page, int f32, hipStream_t st);
+int edge_sm_unrotate_gate(const void* a, const void* gate, int gate_ld, const int* tok_pos, const float* vcs, void* out,
+                          int rows, int HD, int Dv, int f32, hipStream_t st);
 int edge_sm_moe_experts(const void* h, int W, const int* idx, int top, const void* w_gu, const void* w_down, int ff,
                         float limit, int silu, const float* in_w, void* y, void* out, int rows, int E, int f32,
                         hipStream_t st);
@@ -251,8 +263,11 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
                         const at::Tensor& ptab, double scale, int64_t window, int64_t pool, int64_t max_keys,
                         const std::optional<at::Tensor>& seq_start, const std::optional<at::Tensor>& seq_len,
                         const std::optional<at::Tensor>& seq_off, int64_t n, int64_t qtiles, bool chunked, double softcap,
-                        const std::optional<at::Tensor>& slopes, const std::optional<at::Tensor>& sink) {
-  // chunked: `window` is a chunk size and the gate is [T, H * Dv] (see attn_kernel)
+                        const std::optional<at::Tensor>& slopes, const std::optional<at::Tensor>& sink,
+                        int64_t keep_first) {
+  // chunked: `window` is a chunk size and the gate is [T, H * Dv] (see attn_kernel); keep_first: the first
+  // tokens of a sequence that stay visible behind a sliding window
+  TORCH_CHECK(keep_first >= 0 && (keep_first == 0 || (window > 0 && !chunked)), "keep_first goes with a sliding window");
   chk_i32(tok_seq, "tok_seq");
   chk_i32(tok_pos, "tok_pos");
   chk_i32(seq_slot, "seq_slot");
@@ -313,7 +328,7 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
                                           ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)n, (int)qtiles,
                                           (int)H, (int)G, (int)D, (int)Dv, (int)page, PB, (float)scale, (int)window,
                                           PB ? (int)pool : 0, (int)kld, (int)vld, chunked ? 1 : 0, (float)softcap, slopes_p,
-                                          sink_p, gate_elem, stream());
+                                          sink_p, gate_elem, (int)keep_first, stream());
     if (rc != 1) {
       check(rc, "sm_attention_mfma");
       return out;
@@ -322,7 +337,7 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
   // few queries over many keys (decode steps): split every query's keys over several workgroups
   int nsplit = 1;
   {
-    const int64_t vis = (window > 0 ? std::min<int64_t>(window, max_keys) : max_keys) + (PB ? max_keys / pool : 0);
+    const int64_t vis = (window > 0 ? std::min<int64_t>(window + keep_first, max_keys) : max_keys) + (PB ? max_keys / pool : 0);
     const int64_t chunks = (vis + 255) / 256;
     if (T * G <= 64 && chunks > 1) nsplit = (int)std::min<int64_t>(chunks, 8);
   }
@@ -336,7 +351,7 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
                           ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)T, (int)H, (int)G, (int)D, (int)Dv,
                           (int)page, PB, (float)scale, (int)window, PB ? (int)pool : 0, f32(q), nsplit,
                           nsplit > 1 ? part.data_ptr<float>() : nullptr, (int)kld, (int)vld, chunked ? 1 : 0, (float)softcap,
-                          slopes_p, sink_p, gate_elem, stream()), "sm_attention");
+                          slopes_p, sink_p, gate_elem, (int)keep_first, stream()), "sm_attention");
   return out;
 }
 
@@ -619,18 +634,23 @@ at::Tensor sm_delta_scan(const at::Tensor& prep, const at::Tensor& qkv, at::Tens
   return y;
 }
 
+// mode 0: softmax over all experts, the chosen ones renormalised; 1: sigmoid scores; 2: softmax over the chosen logits
 std::tuple<at::Tensor, at::Tensor> sm_moe_route(const at::Tensor& h, const at::Tensor& router, int64_t top, double scale,
-                                                bool sigm) {
+                                                int64_t mode, const std::optional<at::Tensor>& bias) {
   chk_act2(h, "h");
   chk_f32(router, "router");
-  TORCH_CHECK(router.dim() == 2 && router.size(1) == h.size(1), "router: fp32 [E, W]");
+  TORCH_CHECK(router.dim() == 2 && router.size(1) == h.size(1) && mode >= 0 && mode <= 2, "router: fp32 [E, W]");
+  if (bias) {
+    chk_f32(*bias, "bias");
+    TORCH_CHECK(bias->numel() == router.size(0), "bias: fp32 [E]");
+  }
   c10::hip::HIPGuardMasqueradingAsCUDA guard(h.device());
   auto idx = at::empty({h.size(0), top}, h.options().dtype(at::kInt));
   auto wts = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
   auto z = at::empty({h.size(0), router.size(0)}, wts.options());
-  check(edge_sm_moe_route(h.data_ptr(), (int)h.size(1), router.data_ptr<float>(), (int)router.size(0), (int)top, (float)scale,
-                          z.data_ptr<float>(), idx.data_ptr<int>(), wts.data_ptr<float>(), (int)h.size(0), sigm ? 1 : 0,
-                          f32(h), stream()), "sm_moe_route");
+  check(edge_sm_moe_route(h.data_ptr(), (int)h.size(1), router.data_ptr<float>(), bias ? bias->data_ptr<float>() : nullptr,
+                          (int)router.size(0), (int)top, (float)scale, z.data_ptr<float>(), idx.data_ptr<int>(),
+                          wts.data_ptr<float>(), (int)h.size(0), (int)mode, f32(h), stream()), "sm_moe_route");
   return {idx, wts};
 }
 
@@ -735,6 +755,135 @@ at::Tensor sm_delta_prep_head(const at::Tensor& qkv, const at::Tensor& u, int64_
   return prep;
 }
 
+// ---------------------------------------------------------------------------------- residual streams, gated attention
+at::Tensor sm_hyper_read_norm(const at::Tensor& X, const std::optional<at::Tensor>& in_w, const at::Tensor& w, double eps,
+                              bool out_f32) {
+  chk_f32(X, "X");
+  chk_f32(w, "weight");
+  TORCH_CHECK(X.dim() == 3 && w.numel() == X.size(2), "X fp32 [T, S, W], weight [W]");
+  if (in_w) {
+    chk_f32(*in_w, "in_w");
+    TORCH_CHECK(in_w->numel() == X.size(1), "in_w: fp32 [S]");
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(X.device());
+  auto y = at::empty({X.size(0), X.size(2)}, X.options().dtype(act_type(out_f32)));
+  check(edge_sm_hyper_read_norm(X.data_ptr<float>(), in_w ? in_w->data_ptr<float>() : nullptr, w.data_ptr<float>(),
+                                y.data_ptr(), (int)X.size(0), (int)X.size(1), (int)X.size(2), (float)eps, out_f32, stream()),
+        "sm_hyper_read_norm");
+  return y;
+}
+
+void sm_hyper_update(at::Tensor& X, const std::optional<at::Tensor>& mix, const std::optional<at::Tensor>& out_w,
+                     const std::optional<at::Tensor>& y, const std::optional<at::Tensor>& parts,
+                     const std::optional<at::Tensor>& part_w) {
+  chk_f32(X, "X");
+  TORCH_CHECK(X.dim() == 3 && (y || parts) && bool(mix) == bool(out_w), "X fp32 [T, S, W]; y or parts; mix with out_w");
+  const int64_t T = X.size(0), S = X.size(1), W = X.size(2);
+  if (mix) {
+    chk_f32(*mix, "mix");
+    chk_f32(*out_w, "out_w");
+    TORCH_CHECK(mix->numel() == S * S && out_w->numel() == S, "mix fp32 [S, S], out_w fp32 [S]");
+  }
+  int is_f32 = 0, K = 0;
+  if (y) {
+    chk_act2(*y, "y");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == W, "y: [T, W]");
+    is_f32 = f32(*y);
+  }
+  if (parts) {
+    TORCH_CHECK(parts->is_cuda() && parts->is_contiguous() && is_act(*parts) && parts->dim() == 3 && parts->size(0) == T &&
+                    parts->size(2) == W && (!y || parts->scalar_type() == y->scalar_type()), "parts: [T, K, W]");
+    K = (int)parts->size(1);
+    is_f32 = f32(*parts);
+    if (part_w) {
+      chk_f32(*part_w, "part_w");
+      TORCH_CHECK(part_w->numel() == T * K, "part_w: fp32 [T, K]");
+    }
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(X.device());
+  check(edge_sm_hyper_update(X.data_ptr<float>(), mix ? mix->data_ptr<float>() : nullptr,
+                             out_w ? out_w->data_ptr<float>() : nullptr, y ? y->data_ptr() : nullptr,
+                             parts ? parts->data_ptr() : nullptr, parts && part_w ? part_w->data_ptr<float>() : nullptr, K,
+                             (int)T, (int)S, (int)W, is_f32, stream()), "sm_hyper_update");
+}
+
+at::Tensor sm_poly_norm(const at::Tensor& z, const at::Tensor& coef, double eps) {
+  TORCH_CHECK(is_act(z), "z: fp32 / bf16");
+  const int ld = row_ld(z, "z");
+  chk_f32(coef, "coef");
+  TORCH_CHECK(coef.numel() == 4, "coef: fp32 [4]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(z.device());
+  auto y = at::empty({z.size(0), z.size(1)}, z.options());
+  check(edge_sm_poly_norm(z.data_ptr(), ld, coef.data_ptr<float>(), y.data_ptr(), (int)z.size(0), (int)z.size(1), (float)eps,
+                          f32(z), stream()), "sm_poly_norm");
+  return y;
+}
+
+at::Tensor sm_qk_norm_rope_write(const at::Tensor& proj, const at::Tensor& tok_seq, const at::Tensor& tok_pos,
+                                 const at::Tensor& seq_slot, const at::Tensor& ptab, const std::optional<at::Tensor>& qw,
+                                 const std::optional<at::Tensor>& kw, double eps, const std::optional<at::Tensor>& rope,
+                                 const std::optional<at::Tensor>& vrope, const std::optional<at::Tensor>& temp,
+                                 at::Tensor& kp, at::Tensor& vp, int64_t H, int64_t rot) {
+  const int ld = row_ld(proj, "proj");
+  chk_i32(tok_seq, "tok_seq");
+  chk_i32(tok_pos, "tok_pos");
+  chk_i32(seq_slot, "seq_slot");
+  chk_table(ptab);
+  TORCH_CHECK(is_act(proj) && kp.scalar_type() == proj.scalar_type() && kp.is_cuda() && kp.is_contiguous() && kp.dim() == 4 &&
+                  vp.scalar_type() == proj.scalar_type() && vp.is_cuda() && vp.is_contiguous() && vp.dim() == 4 &&
+                  vp.size(0) == kp.size(0) && vp.size(1) == kp.size(1) && vp.size(2) == kp.size(2),
+              "pages: [pages, page, G, D] and [pages, page, G, Dv] in proj's dtype");
+  const int64_t T = proj.size(0), page = kp.size(1), G = kp.size(2), D = kp.size(3), Dv = vp.size(3);
+  TORCH_CHECK(proj.size(1) >= (H + G) * D + G * Dv, "proj: [T, (H + G) D + G Dv + ..]");
+  TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T, "token metadata: [T]");
+  auto table = [&](const std::optional<at::Tensor>& t, int64_t dims, const char* name) -> const float* {
+    if (!t) return nullptr;
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat && t->is_contiguous() && t->dim() == 3 &&
+                    t->size(1) * 2 == dims && t->size(2) == 2, name, ": fp32 [pos, dims / 2, 2]");
+    return t->data_ptr<float>();
+  };
+  auto vec = [&](const std::optional<at::Tensor>& t, int64_t n, const char* name) -> const float* {
+    if (!t) return nullptr;
+    chk_f32(*t, name);
+    TORCH_CHECK(t->numel() == n, name, ": wrong size");
+    return t->data_ptr<float>();
+  };
+  TORCH_CHECK(rot == 0 || rope, "rope table missing");
+  const float* cs = rot > 0 ? table(rope, rot, "rope") : nullptr;
+  const float* vcs = table(vrope, Dv, "value rope");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(proj.device());
+  auto q = at::empty({T, H, D}, proj.options());
+  check(edge_sm_qk_norm_rope_write(proj.data_ptr(), ld, tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(),
+                                   seq_slot.data_ptr<int>(), ptab.data_ptr<int>(), (int)ptab.stride(0), vec(qw, D, "q norm"),
+                                   vec(kw, D, "k norm"), (float)eps, cs, vcs, vec(temp, H, "temp"), q.data_ptr(),
+                                   kp.data_ptr(), vp.data_ptr(), (int)T, (int)H, (int)G, (int)D, (int)Dv, (int)rot, (int)page,
+                                   f32(proj), stream()), "sm_qk_norm_rope_write");
+  return q;
+}
+
+at::Tensor sm_unrotate_gate(const at::Tensor& a, const std::optional<at::Tensor>& gate, const at::Tensor& tok_pos,
+                            const std::optional<at::Tensor>& vrope, int64_t H) {
+  chk_act2(a, "a");
+  chk_i32(tok_pos, "tok_pos");
+  const int64_t T = a.size(0), HD = a.size(1);
+  TORCH_CHECK(H > 0 && HD % H == 0 && tok_pos.numel() == T, "a: [T, H Dv], tok_pos [T]");
+  const int64_t Dv = HD / H;
+  int gate_ld = 0;
+  if (gate) {
+    gate_ld = row_ld(*gate, "gate");
+    TORCH_CHECK(gate->size(0) == T && gate->size(1) == HD && gate->scalar_type() == a.scalar_type(), "gate: [T, H Dv]");
+  }
+  if (vrope)
+    TORCH_CHECK(vrope->is_cuda() && vrope->scalar_type() == at::kFloat && vrope->is_contiguous() && vrope->dim() == 3 &&
+                    vrope->size(1) * 2 == Dv && vrope->size(2) == 2, "value rope: fp32 [pos, Dv / 2, 2]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  auto out = at::empty_like(a);
+  check(edge_sm_unrotate_gate(a.data_ptr(), gate ? gate->data_ptr() : nullptr, gate_ld, tok_pos.data_ptr<int>(),
+                              vrope ? vrope->data_ptr<float>() : nullptr, out.data_ptr(), (int)T, (int)HD, (int)Dv, f32(a),
+                              stream()), "sm_unrotate_gate");
+  return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -765,4 +914,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("sm_group_norm_residual", &sm_group_norm_residual);
   m.def("sm_glu_silu", &sm_glu_silu);
   m.def("sm_delta_prep_head", &sm_delta_prep_head);
+  m.def("sm_hyper_read_norm", &sm_hyper_read_norm);
+  m.def("sm_hyper_update", &sm_hyper_update);
+  m.def("sm_poly_norm", &sm_poly_norm);
+  m.def("sm_qk_norm_rope_write", &sm_qk_norm_rope_write);
+  m.def("sm_unrotate_gate", &sm_unrotate_gate);
 }

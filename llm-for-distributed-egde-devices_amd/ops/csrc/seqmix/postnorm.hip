@@ -382,7 +382,7 @@ __global__ void __launch_bounds__(NT) delta_scan_kernel(const float* __restrict_
 // Router scores: one wave per (token, expert), fp32 dot product over the width with 8-element loads.
 template <typename T>
 __global__ void __launch_bounds__(NT) moe_logits_kernel(const T* __restrict__ h, int W, const float* __restrict__ router,
-                                                        int E, float* __restrict__ z) {
+                                                        int E, float* __restrict__ z, const float* __restrict__ bias) {
   const size_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, e = blockIdx.y * (NT / 64) + (threadIdx.x >> 6);
   if (e >= E) return;
@@ -401,13 +401,13 @@ __global__ void __launch_bounds__(NT) moe_logits_kernel(const T* __restrict__ h,
     for (int c = lane; c < W; c += 64) acc += ldf<T>(hr + c) * rr[c];
   }
   acc = wave_sum(acc);
-  if (lane == 0) z[t * E + e] = acc;
+  if (lane == 0) z[t * E + e] = acc + (bias ? bias[e] : 0.f);
 }
 
 // One wave per token: softmax over the experts' scores, then the `top` largest (lowest index on a tie),
 // divided by their sum (+ 1e-20) and multiplied by scale.  sigm: the scores are sigmoid(z) and the `top`
 // largest keep their own value (times scale); they are picked by z itself (the same order), so scores that
-// round to 1 do not tie.
+// round to 1 do not tie.  sigm == 2: the `top` largest logits, softmax over those alone (times scale).
 __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ z, int E, int top, float scale,
                                                       int* __restrict__ idx, float* __restrict__ wts, int sigm) {
   extern __shared__ __attribute__((aligned(16))) float z_s[];   // [E]
@@ -444,9 +444,14 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
     if (lane == 0) z_s[bi] = gone;                           // LDS accesses of one wave keep their order
     tot += best;
   }
+  float soft = 0.f;
+  if (sigm == 2) {                                           // the first choice holds the largest logit
+    const float ex = lane < top ? expf(my_w - __shfl(my_w, 0, 64)) : 0.f;
+    soft = ex / wave_sum(ex);
+  }
   if (lane < top) {
     idx[t * top + lane] = my_i;
-    wts[t * top + lane] = sigm ? sigmoidf_(my_w) * scale : my_w / (tot + 1e-20f) * scale;
+    wts[t * top + lane] = sigm == 2 ? soft * scale : sigm ? sigmoidf_(my_w) * scale : my_w / (tot + 1e-20f) * scale;
   }
 }
 
@@ -636,12 +641,12 @@ int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, 
 }
 
 // z: fp32 scratch [rows, E] (the experts' scores)
-int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, float* z, int* idx, float* wts,
-                      int rows, int sigm, int f32, hipStream_t st) {
+int edge_sm_moe_route(const void* h, int W, const float* router, const float* bias, int E, int top, float scale, float* z,
+                      int* idx, float* wts, int rows, int sigm, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   if (top < 1 || top > E || top > 64 || E > 8192) return -2;
   SM_T(f32, hipLaunchKernelGGL(moe_logits_kernel<T>, dim3(rows, (E + NT / 64 - 1) / (NT / 64)), dim3(NT), 0, st, (const T*)h,
-                               W, router, E, z));
+                               W, router, E, z, bias));
   hipLaunchKernelGGL(moe_topk_kernel, dim3(rows), dim3(64), (size_t)E * 4, st, (const float*)z, E, top, scale, idx, wts, sigm);
   return (int)hipGetLastError();
 }

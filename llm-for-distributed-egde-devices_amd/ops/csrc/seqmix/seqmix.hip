@@ -344,7 +344,8 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
                                                   int page, int PB, float scale, int window, int pool, int nsp, int nsplit,
                                                   float* __restrict__ part, int kld, int vld, int chunked, float cap,
                                                   const float* __restrict__ slopes, const float* __restrict__ sink,
-                                                  int gate_elem) {
+                                                  int gate_elem, int keep_first) {
+  // keep_first: the tokens j < keep_first stay visible behind a sliding window
   // chunked: `window` is a chunk size (query i sees floor(i / window) * window .. i); cap / slopes: see attn_chunk;
   // sink: a number per query head that joins the softmax denominator (it enters as the first key split's
   // starting maximum with sum 1 and no value); gate_elem: the gate is [T, H * Dv], one per output coordinate
@@ -387,10 +388,18 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
   const int jlo = window > 0 ? (chunked ? (i / window) * window : max(0, i - window + 1)) : 0;
   const int nt = i - jlo + 1;
   const int nb = (!chunked && window > 0 && pool > 0 && i - window + 1 > 0) ? (i - window + 1) / pool : 0;
+  const int kf = (!chunked && window > 0) ? min(keep_first, jlo) : 0;   // kept first tokens that lie before the window
   // key chunks [ci0, ci1) of this query belong to this workgroup (blockIdx.z of nsplit; 1: all of them)
-  const int nchunks = (nt + KC - 1) / KC + (nb + KC - 1) / KC, cps = (nchunks + nsplit - 1) / nsplit;
+  const int nchunks = (kf + KC - 1) / KC + (nt + KC - 1) / KC + (nb + KC - 1) / KC, cps = (nchunks + nsplit - 1) / nsplit;
   const int ci0 = blockIdx.z * cps, ci1 = min(nchunks, ci0 + cps);
   int ci = 0;
+  for (int c0 = 0; c0 < kf; c0 += KC, ++ci) {
+    if (ci < ci0 || ci >= ci1) continue;
+    const int j = c0 + tid;
+    const int rowidx = j < kf ? pt[j / page] * page + j % page : 0;
+    attn_chunk<T, RMAX, DVL, VEC>(kp, vp, min(KC, kf - c0), g, kld, vld, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc,
+                                  cap, slopes ? sl_s : nullptr, i - j);
+  }
   for (int c0 = 0; c0 < nt; c0 += KC, ++ci) {
     if (ci < ci0 || ci >= ci1) continue;
     const int j = jlo + c0 + tid;
@@ -489,13 +498,14 @@ constexpr int MQ = 64, MK = 64;
 // 1024 workgroups of a 4096-token, 16-head prompt are resident at once)
 // KVS: the value of a cached row is its first Dv numbers (a latent cache, or values that are the keys): the
 // staged key tile serves as the value tile, nothing is loaded twice
-// EXT: scores are capped (cap tanh(s / cap), cap > 0) and lose slopes[head] * distance; `window` is a chunk
-// size (a query sees its own chunk's start .. itself); sink[head] joins the softmax denominator; the gate
-// is [T, H * Dv], one per output coordinate
+// EXT: scores are capped (cap tanh(s / cap), cap > 0) and lose slopes[head] * distance; chunked: `window` is a
+// chunk size (a query sees its own chunk's start .. itself), else a sliding window beside the sequence's first
+// keep_first tokens; sink[head] joins the softmax denominator; the gate is [T, H * Dv], one per output coordinate
 struct AttnExt {
   float scale, cap;
   const float* slopes;
   const float* sink;
+  int chunked, keep_first;
 };
 
 template <int DK, int DV, int RH, bool KVS, bool EXT = false>
@@ -560,7 +570,10 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
   if constexpr (EXT) {
     if (window > 0) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) clo[i] = ((start + wq0 + 4 * g4 + i) / window) * window;
+      for (int i = 0; i < 4; ++i) {
+        const int qpos = start + wq0 + 4 * g4 + i;
+        clo[i] = ext.chunked ? (qpos / window) * window : max(0, qpos - window + 1);
+      }
     }
 #pragma unroll
     for (int r = 0; r < RH; ++r) {
@@ -572,9 +585,14 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
     }
   }
   const int imin = start + qt * MQ, imax = start + min(len, qt * MQ + MQ) - 1;
-  const int jlo = window > 0 ? (EXT ? (imin / window) * window : max(0, imin - window + 1)) : 0;
+  const int jlo = window > 0 ? ((EXT && ext.chunked) ? (imin / window) * window : max(0, imin - window + 1)) : 0;
   const int nbmax = (window > 0 && pool > 0 && imax - window + 1 > 0) ? (imax - window + 1) / pool : 0;
-  const int tok_tiles = imax / MK - jlo / MK + 1, ntiles = tok_tiles + (nbmax + MK - 1) / MK;
+  // the tiles that hold kept first tokens and lie wholly before the window's first tile come first
+  const int nfirst = (EXT && window > 0 && !ext.chunked) ? min((ext.keep_first + MK - 1) / MK, jlo / MK) : 0;
+  const int tok_tiles = nfirst + imax / MK - jlo / MK + 1, ntiles = tok_tiles + (nbmax + MK - 1) / MK;
+  auto tile_base = [&](int tile) {                           // first position (token tiles) / block (pooled tiles) of a tile
+    return tile < nfirst ? tile * MK : tile < tok_tiles ? (jlo / MK + tile - nfirst) * MK : (tile - tok_tiles) * MK;
+  };
   for (int i = tid; i < min(imax / MK + 1, NPID); i += NT) pid_s[i] = pt[i];
   __syncthreads();
   auto page_of = [&](int idx) { return idx < NPID ? pid_s[idx] : pt[idx]; };
@@ -586,7 +604,7 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
   uint4 kreg[KL], vreg[VL > 0 ? VL : 1];
   auto load_tile = [&](int tile) {
     const bool tok = tile < tok_tiles;
-    const int base = tok ? (jlo / MK + tile) * MK : (tile - tok_tiles) * MK;
+    const int base = tile_base(tile);
     const size_t prow = tok ? (size_t)page_of(base / MK) * MK : 0;
 #pragma unroll
     for (int i = 0; i < KL + VL; ++i) {
@@ -623,7 +641,7 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
   if (ntiles > 0) load_tile(0);
   for (int tile = 0; tile < ntiles; ++tile) {
     const bool tok = tile < tok_tiles;
-    const int base = tok ? (jlo / MK + tile) * MK : (tile - tok_tiles) * MK;   // first position / block of the tile
+    const int base = tile_base(tile);
     __syncthreads();                                         // every wave is done with the previous tile
     store_tile();
     __syncthreads();
@@ -653,7 +671,7 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
         bool vis;
         float v;
         if constexpr (EXT) {
-          vis = key <= qpos && key >= clo[i];
+          vis = key <= qpos && (key >= clo[i] || key < ext.keep_first);
           const float bias = sl2[r] * (float)(qpos - key);
           if (ext.cap > 0.f)                                 // 2^(xs s) = inf gives the cap itself, 0 gives -cap
             v = c1 - c2 * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(sc[nt][i] * xs) + 1.f) - bias;
@@ -1227,9 +1245,9 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
                       int window, int pool, int f32, int nsplit, float* part, int kld, int vld, int chunked, float cap,
-                      const float* slopes, const float* sink, int gate_elem, hipStream_t st) {
+                      const float* slopes, const float* sink, int gate_elem, int keep_first, hipStream_t st) {
   if (rows == 0) return 0;
-  if (G <= 0 || H % G || Dv > 512 || (chunked && pool > 0)) return -2;
+  if (G <= 0 || H % G || Dv > 512 || (chunked && pool > 0) || keep_first < 0) return -2;
   const int R = H / G;
   const int rmax = edge_sm_attention_rmax(rows, H, G, D, Dv);
   if (rmax == 0) return -3;
@@ -1241,7 +1259,7 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
   SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL, V>), dim3(rows, G * nsp, nsplit), dim3(NT), lds, st, (const T*)q,         \
                                (const T*)gate, gate_ld, (const T*)kp, (const T*)vp, kb, vb, tok_seq, tok_pos,       \
                                seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool, nsp, nsplit, part, \
-                               kld, vld, chunked, cap, slopes, sink, gate_elem))
+                               kld, vld, chunked, cap, slopes, sink, gate_elem, keep_first))
 #define SM_ATT(RM, DL)               \
   do {                               \
     if (vec) SM_ATT_V(RM, DL, true); \
@@ -1336,9 +1354,9 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
                            const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
                            int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
                            int pool, int kld, int vld, int chunked, float cap, const float* slopes, const float* sink,
-                           int gate_elem, hipStream_t st) {
+                           int gate_elem, int keep_first, hipStream_t st) {
   if (page != MK || G <= 0 || H % G || kld % 8 || vld % 8) return 1;
-  const bool extras = chunked || cap > 0.f || slopes || sink || gate_elem;
+  const bool extras = chunked || cap > 0.f || slopes || sink || gate_elem || keep_first > 0;
   if (n == 0 || qtiles == 0) return 0;
   const float sl2 = scale * 1.4426950408889634f;
   // query heads per workgroup: a staged tile can serve 4 or 2 heads of a kv group, but the kernel is
@@ -1352,11 +1370,12 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
   const bool kvs = kp == vp && kld == vld;
   if (kvs && pool > 0) return 1;                             // pooled entries keep separate key / value rows
   if (extras) {
-    // the capped / biased / chunked form: values that are the keys, an element-wise gate or none
-    if (!kvs || D != Dv || pool > 0 || (window > 0 && !chunked) || (gate && !gate_elem)) return 1;
-    const AttnExt ext{scale, cap, slopes, sink};
-#define SM_MFX_R(DK, DV, RH)                                                                                         \
-  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV, RH, true, true>), dim3(qtiles, H / RH), dim3(NT), 0, st,              \
+    // the capped / biased / chunked / sink / kept-first-tokens form: an element-wise gate or none, no pooled blocks
+    if ((kvs && D != Dv) || pool > 0 || (gate && !gate_elem)) return 1;
+    const AttnExt ext{scale, cap, slopes, sink, chunked, (chunked || window <= 0) ? 0 : keep_first};
+#define SM_MFX_R(DK, DV, RH) SM_MFX_RK(DK, DV, RH, true)
+#define SM_MFX_RK(DK, DV, RH, KVS)                                                                                   \
+  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV, RH, KVS, true>), dim3(qtiles, H / RH), dim3(NT), 0, st,               \
                      (const bf16_t*)q, (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb,   \
                      seq_slot, seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window,   \
                      pool, kld, vld, ext)
@@ -1366,13 +1385,30 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
     else if (rh == 2) SM_MFX_R(DK, DV, 2);\
     else SM_MFX_R(DK, DV, 1);             \
   } while (0)
-    if (D == 32) SM_MFX(1, 2);
-    else if (D == 64) SM_MFX(2, 4);
-    else if (D == 96) SM_MFX(3, 6);
-    else if (D == 128) SM_MFX(4, 8);
-    else if (D == 256) SM_MFX_R(8, 16, 1);
+#define SM_MFXS(DK, DV)                          \
+  do {                                           \
+    if (rh == 4) SM_MFX_RK(DK, DV, 4, false);    \
+    else if (rh == 2) SM_MFX_RK(DK, DV, 2, false);\
+    else SM_MFX_RK(DK, DV, 1, false);            \
+  } while (0)
+    if (kvs) {
+      if (D == 32) SM_MFX(1, 2);
+      else if (D == 64) SM_MFX(2, 4);
+      else if (D == 96) SM_MFX(3, 6);
+      else if (D == 128) SM_MFX(4, 8);
+      else if (D == 256) SM_MFX_R(8, 16, 1);
+      else return 1;
+    }
+    else if (D == 64 && Dv == 64) SM_MFXS(2, 4);             // separate key and value pages
+    else if (D == 96 && Dv == 96) SM_MFXS(3, 6);
+    else if (D == 128 && Dv == 128) SM_MFXS(4, 8);
+    else if (D == 128 && Dv == 64) SM_MFXS(4, 4);
+    else if (D == 64 && Dv == 128) SM_MFXS(2, 8);
+    else if (D == 32 && Dv == 32) SM_MFXS(1, 2);
     else return 1;
+#undef SM_MFXS
 #undef SM_MFX
+#undef SM_MFX_RK
 #undef SM_MFX_R
     return (int)hipGetLastError();
   }

@@ -239,10 +239,13 @@ ATTN_MFMA_MIN = int(__import__("os").environ.get("EDGELLM_ATTN_MFMA_MIN", "16"))
 
 
 def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages, v_pages, k_pool, v_pool,
-                          meta: RaggedMeta, scale: float, window: Optional[int], pool: Optional[int]) -> torch.Tensor:
+                          meta: RaggedMeta, scale: float, window: Optional[int], pool: Optional[int],
+                          sink: Optional[torch.Tensor] = None, keep_first: int = 0) -> torch.Tensor:
     """q [T, H, D] -> [T, H * Dv].  Query position i sees the tokens j with 0 <= i - j < window and
     the pooled blocks b with b pool + pool - 1 <= i - window, in one softmax (fp32); head h's result
-    is multiplied by sigmoid(gate[t, h]) when ``gate`` ([T, H] view) is given."""
+    is multiplied by sigmoid(gate[t, h]) when ``gate`` ([T, H] view) is given.  ``keep_first``: the
+    tokens j < keep_first stay visible behind the window (j <= i).  ``sink`` (fp32 [H]): exp(sink[h])
+    joins head h's softmax denominator; it has no value."""
     T, H, D = q.shape
     G, Dv = k_pages.shape[2], v_pages.shape[3]
     if _gpu(q):
@@ -255,7 +258,7 @@ def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages
                                    meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.page_table, float(scale),
                                    int(window) if window is not None else 0, int(pool or 0), int(meta.max_keys),
                                    meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n), int(qtiles), False, 0.0,
-                                   None, None)
+                                   None, sink, int(keep_first if window is not None else 0))
     page = meta.page
     out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
     R = H // G
@@ -271,7 +274,7 @@ def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages
         d = i[:, None] - pos[None]
         vis = d >= 0
         if window is not None:
-            vis &= d < window
+            vis &= (d < window) | (pos[None] < keep_first)
         s = s.masked_fill(~vis[:, None, None, :], float("-inf"))
         vals = v
         if window is not None and pool:
@@ -286,7 +289,9 @@ def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages
                 sb = sb.masked_fill(~seen[:, None, None, :], float("-inf"))
                 s = torch.cat([s, sb], -1)
                 vals = torch.cat([v, vb], 0)
-        p = torch.softmax(s, -1)
+        if sink is not None:
+            s = torch.cat([s, sink.float().view(1, G, R, 1).expand(n, G, R, 1)], -1)
+        p = torch.softmax(s, -1)[..., :vals.shape[0]]
         out[off:off + n] = torch.einsum("ngrl,lgd->ngrd", p, vals).reshape(n, H, Dv)
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[..., None]
@@ -316,7 +321,7 @@ def chunk_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages: torc
         return _ext().sm_attention(q, gate, k_pages, k_pages, None, None, meta.tok_seq, meta.tok_pos, meta.seq_slot,
                                    meta.page_table, float(scale), int(chunk or 0), 0, int(meta.max_keys), meta.seq_start,
                                    meta.seq_len, meta.seq_off, int(meta.n), int(qtiles), True, float(softcap or 0.0),
-                                   slopes, sink)
+                                   slopes, sink, 0)
     page, R = meta.page, H // G
     out = torch.empty(T, H, D, dtype=torch.float32, device=q.device)
     for slot, start, n, off in meta.host:
@@ -661,14 +666,22 @@ def head_norm_gate(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, heads
 
 
 # --------------------------------------------------------------------------- mixture of experts
-def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, mode: str = "softmax"):
-    """Router in fp32 over h [T, W] (router fp32 [E, W]).  ``mode`` "softmax": the ``top`` largest
-    softmax scores of every token, divided by their sum (+ 1e-20) and multiplied by ``scale``;
-    "sigmoid": the ``top`` largest of sigmoid(logit) as they are, times ``scale``.  Returns (expert ids
-    int32 [T, top], weights fp32 [T, top]), largest first (the lower id on a tie)."""
+def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, mode: str = "softmax",
+              bias: Optional[torch.Tensor] = None):
+    """Router in fp32 over h [T, W] (router fp32 [E, W], logits W_r h + ``bias`` fp32 [E]).  ``mode``
+    "softmax": the ``top`` largest softmax scores of every token, divided by their sum (+ 1e-20) and
+    multiplied by ``scale``; "sigmoid": the ``top`` largest of sigmoid(logit) as they are, times ``scale``;
+    "top_softmax": the ``top`` largest logits, softmax over those alone, times ``scale``.  Returns
+    (expert ids int32 [T, top], weights fp32 [T, top]), largest first (the lower id on a tie)."""
     if _gpu(h):
-        return _ext().sm_moe_route(h, router, int(top), float(scale), mode == "sigmoid")
+        return _ext().sm_moe_route(h, router, int(top), float(scale), {"softmax": 0, "sigmoid": 1, "top_softmax": 2}[mode],
+                                   bias)
     z = h.float() @ router.float().t()
+    if bias is not None:
+        z = z + bias.float()
+    if mode == "top_softmax":
+        zt, idx = torch.topk(z, top, -1)
+        return idx.int(), torch.softmax(zt, -1) * scale
     if mode == "sigmoid":                                        # picked by the logits: scores that round to 1 do not tie
         zt, idx = torch.topk(z, top, -1)
         return idx.int(), torch.sigmoid(zt) * scale
@@ -737,3 +750,101 @@ def _moe_experts_sorted(h, idx, w_gu, w_down, limit, act="glu_clamp", in_w=None)
     back = torch.empty_like(order)
     back[order] = torch.arange(T * top, device=h.device)
     return o.index_select(0, back).view(T, top, -1)
+
+
+# --------------------------------------------------------------------------- residual streams
+def hyper_read_norm(X: torch.Tensor, in_w: Optional[torch.Tensor], weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """X fp32 [T, S, W] (S copies of the residual stream) -> RMS norm of u = sum_s in_w[s] X[:, s]
+    (``in_w`` fp32 [S]; None: the plain sum) times weight [W], stored as ``out_dtype`` [T, W]."""
+    if _gpu(X):
+        return _ext().sm_hyper_read_norm(X, in_w, weight, float(eps), out_dtype == torch.float32)
+    u = X.sum(1) if in_w is None else torch.einsum("s,tsw->tw", in_w.float(), X)
+    return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
+
+
+def hyper_update(X: torch.Tensor, mix: Optional[torch.Tensor], out_w: Optional[torch.Tensor], y: Optional[torch.Tensor],
+                 parts: Optional[torch.Tensor] = None, part_w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """X fp32 [T, S, W], in place, all streams at once from the old ones:
+    X[:, r] <- sum_s mix[s, r] X[:, s] + out_w[r] v, with v = y + sum_k part_w[:, k] parts[:, k] summed in
+    fp32 in k order (``y`` [T, W] or None; ``parts`` [T, K, W] with ``part_w`` fp32 [T, K]: a mixture's
+    expert outputs).  ``mix`` fp32 [S, S] indexed [from, to] and ``out_w`` fp32 [S]; both None: X += v."""
+    if _gpu(X):
+        _ext().sm_hyper_update(X, mix, out_w, y, parts, part_w)
+        return X
+    v = y.float() if y is not None else torch.zeros_like(X[:, 0])
+    if parts is not None:
+        for k in range(parts.shape[1]):
+            v = v + (parts[:, k].float() if part_w is None else part_w[:, k:k + 1] * parts[:, k].float())
+    if mix is None:
+        X.add_(v[:, None, :])
+    else:
+        X.copy_(torch.einsum("sr,tsw->trw", mix.float(), X) + out_w.float()[None, :, None] * v[:, None, :])
+    return X
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """z [T, F] -> a N(z) + b N(z^2) + c N(z^3) + e with (a, b, c, e) = ``coef`` (fp32 [4]), powers
+    taken element by element and N(v) = v / sqrt(mean(v^2) + eps) over the row (fp32 math, stored in z's dtype)."""
+    if _gpu(z):
+        return _ext().sm_poly_norm(z, coef, float(eps))
+    x = z.float()
+    N = lambda v: v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    c = coef.float()
+    return (c[0] * N(x) + c[1] * N(x * x) + c[2] * N(x * x * x) + c[3]).to(z.dtype)
+
+
+# --------------------------------------------------------------------------- gated attention
+def qk_norm_rope_write(proj: torch.Tensor, meta: RaggedMeta, q_w: Optional[torch.Tensor], k_w: Optional[torch.Tensor],
+                       eps: float, rope: Optional[torch.Tensor], v_rope: Optional[torch.Tensor], temp: Optional[torch.Tensor],
+                       k_pages: torch.Tensor, v_pages: torch.Tensor, heads: int, rot_dims: int) -> torch.Tensor:
+    """proj [T, q | k | v | ...] -> q [T, heads, D]; keys and values go to their pages at each token's
+    position.  In fp32, per head: q and k are divided by their root mean square over D (eps inside the
+    root) times ``q_w`` / ``k_w`` (fp32 [D]; None: no norm), then the pairs (2i, 2i + 1), i < rot_dims / 2,
+    are turned by ``rope[pos, i]`` = (cos, sin); q is multiplied by ``temp[h]`` (fp32 [heads]; None: 1).
+    The values' pairs (2m, 2m + 1) over all Dv coordinates are turned by ``v_rope[pos, m]`` (None: stored
+    as they are)."""
+    G, D, Dv = k_pages.shape[2], k_pages.shape[3], v_pages.shape[3]
+    if _gpu(proj):
+        return _ext().sm_qk_norm_rope_write(proj, meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.page_table, q_w, k_w,
+                                            float(eps), rope if rot_dims else None, v_rope, temp, k_pages, v_pages,
+                                            int(heads), int(rot_dims))
+    T = proj.shape[0]
+    x = proj.float()
+    q = x[:, :heads * D].view(T, heads, D)
+    k = x[:, heads * D:(heads + G) * D].view(T, G, D)
+    v = x[:, (heads + G) * D:(heads + G) * D + G * Dv].view(T, G, Dv)
+    pos = meta.tok_pos.long()
+    if q_w is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_w.float()
+    if k_w is not None:
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_w.float()
+    if rope is not None and rot_dims:
+        cs = rope[pos][:, None]
+        q, k = _rotate_pairs(q, cs, rot_dims), _rotate_pairs(k, cs, rot_dims)
+    if temp is not None:
+        q = q * temp.float()[None, :, None]
+    if v_rope is not None:
+        v = _rotate_pairs(v, v_rope[pos][:, None], Dv)
+    slot = meta.seq_slot.long()[meta.tok_seq.long()]
+    pid = meta.page_table[slot, pos // meta.page].long()
+    k_pages[pid, pos % meta.page] = k.to(k_pages.dtype)
+    v_pages[pid, pos % meta.page] = v.to(v_pages.dtype)
+    return q.to(proj.dtype)
+
+
+def unrotate_gate(a: torch.Tensor, gate: Optional[torch.Tensor], meta: RaggedMeta, v_rope: Optional[torch.Tensor],
+                  heads: int) -> torch.Tensor:
+    """a [T, heads * Dv] (each head's weighted sum of rotated values) -> every head's pairs (2m, 2m + 1)
+    turned back by the token's own position (``v_rope[pos, m]`` = (cos, sin), applied with -sin; None: as it
+    is), then times sigmoid(gate) element by element (``gate`` [T, heads * Dv], a possibly strided view; None: 1)."""
+    if _gpu(a):
+        return _ext().sm_unrotate_gate(a, gate, meta.tok_pos, v_rope, int(heads))
+    T = a.shape[0]
+    o = a.float().view(T, heads, -1)
+    if v_rope is not None:
+        cs = v_rope[meta.tok_pos.long()][:, None]
+        o = _rotate_pairs(o, torch.stack([cs[..., 0], -cs[..., 1]], -1), o.shape[-1])
+    o = o.reshape(T, -1)
+    if gate is not None:
+        o = o * torch.sigmoid(gate.float())
+    return o.to(a.dtype)
