@@ -559,7 +559,7 @@ at::Tensor sm_latent_write(const std::optional<at::Tensor>& u, int64_t c0, const
   chk_table(ptab);
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && is_act(q), "q: [T, H, D + R]");
   TORCH_CHECK(pages.is_cuda() && pages.is_contiguous() && pages.dim() == 4 && pages.size(2) == 1 &&
-                  pages.scalar_type() == q.scalar_type() && pages.size(3) > kvr, "pages: [pages, page, 1, kv_rank + R]");
+                  pages.scalar_type() == q.scalar_type() && pages.size(3) >= kvr, "pages: [pages, page, 1, kv_rank + R]");
   const int64_t T = q.size(0), H = q.size(1), R = pages.size(3) - kvr, D = q.size(2) - R, page = pages.size(1);
   TORCH_CHECK(D >= 0 && q_lat.is_cuda() && q_lat.dim() == 3 && q_lat.size(0) == T && q_lat.size(1) == H &&
                   q_lat.size(2) == kvr && q_lat.stride(2) == 1 && q_lat.scalar_type() == q.scalar_type(),
