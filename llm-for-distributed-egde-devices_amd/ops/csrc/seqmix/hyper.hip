@@ -11,7 +11,7 @@
 
 namespace {
 
-constexpr int MAXS = 8;                                      // residual streams
+constexpr int MAXS = 16;                                     // residual streams
 
 // X [rows, S, W] fp32; u = sum_s in_w[s] X[t, s] (in_w null: the plain sum); y = u / sqrt(mean(u^2) + eps) * w.
 // LDS: u [W].  VEC (W % 4 == 0): four coordinates per thread and pass.

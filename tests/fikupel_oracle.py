@@ -77,7 +77,7 @@ def latent_attention(h, w, p, m, eps):
     for i in range(T):
         lo = 0 if win is None else max(0, i - win + 1)
         for hh in range(H):
-            s = np.array([q[i, hh] @ k[j, hh] for j in range(lo, i + 1)]) * m["scale"]
+            s = (k[lo:i + 1, hh] @ q[i, hh]) * m["scale"]
             pw = softmax_with_sink(s, None if sink is None else float(sink[hh]))
             out[i, hh] = pw @ v[lo:i + 1, hh]
     return out.reshape(T, H * Dv) @ w[p + "o"].T
@@ -92,8 +92,9 @@ def gated_attention(h, w, p, m, eps):
     q = (h @ w[p + "q"].T).reshape(T, H, D)
     k = (h @ w[p + "k"].T).reshape(T, G, D)
     v = (h @ w[p + "v"].T).reshape(T, G, Dv)
-    q = rms(q, eps) * w[p + "q.norm"]
-    k = rms(k, eps) * w[p + "k.norm"]
+    if p + "q.norm" in w:
+        q = rms(q, eps) * w[p + "q.norm"]
+        k = rms(k, eps) * w[p + "k.norm"]
     if rot:
         fk = pair_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
         fv = pair_frequencies(Dv, rot["base"])
@@ -109,7 +110,7 @@ def gated_attention(h, w, p, m, eps):
         seen = [j for j in range(i + 1) if win is None or i - j < win or j < keep]
         for hh in range(H):
             g = hh // (H // G)
-            s = np.array([q[i, hh] @ k[j, g] for j in seen]) * m["scale"]
+            s = (k[seen, g] @ q[i, hh]) * m["scale"]
             if temp is not None:
                 s = s * temp[hh]
             pw = softmax_with_sink(s, None if sink is None else float(sink[hh]))
