@@ -102,11 +102,13 @@ def parse(argv=None):
     ap.add_argument("--hybrid-compare", action="store_true",
                     help="instead of the headline workload: prefill / decode throughput of the Nudadra layer-spec "
                          "model beside the parallel-residual decoder of equal size (one JSON line)")
-    ap.add_argument("--hybrid-family", default="nudadra", choices=["nudadra", "pagonex", "vetevik"],
+    ap.add_argument("--hybrid-family", default="nudadra", choices=["nudadra", "pagonex", "vetevik", "fikupel"],
                     help="with --hybrid-compare: nudadra (beside the parallel-residual decoder), pagonex (latent "
                          "attention + gated delta rule + mixture of experts, beside the Nudadra hybrid) or vetevik "
                          "(chunked attention with a sink + per-head-decay delta rule + sigmoid-routed experts, beside "
-                         "the Pagonex model)")
+                         "the Pagonex model) or fikupel (latent attention without positions + gated attention with "
+                         "rotated values, windows and sinks, PolyNorm / expert feed-forwards over two residual streams, "
+                         "beside the Vetevik model)")
     ap.add_argument("--hybrid-sizes", default="w1024,w2048", help="comma list of w1024 | w2048 | w4096")
     ap.add_argument("--hybrid-prompt", type=int, default=4096)
     ap.add_argument("--hybrid-batch", type=int, default=4)

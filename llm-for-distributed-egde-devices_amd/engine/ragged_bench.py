@@ -5,7 +5,11 @@ mixture-of-experts feed-forwards) beside the Nudadra hybrid, its closest relativ
 windowed attention over the paged cache, a recurrent mixer and a feed-forward per layer; or
 (``--hybrid-family vetevik``) the Vetevik model (chunked attention whose values are its keys, a gated
 delta rule with per-head decays, sigmoid-routed experts, norms on both sides of every sublayer)
-beside the Pagonex model of equal width, heads, state size and active expert width.
+beside the Pagonex model of equal width, heads, state size and active expert width; or
+(``--hybrid-family fikupel``) the Fikupel model (latent attention without positions and gated
+grouped-query attention with rotated values, both with a window and a sink, PolyNorm and expert
+feed-forwards, two residual streams) beside the Vetevik model of equal width, heads, head size, window
+and active expert width.
 
 Sizes resemble real layers (random weights): the hybrid layer has windowed attention with pooled
 blocks + a Mamba-2 mixer + a squared-ReLU feed-forward; the comparison model is the
@@ -24,8 +28,8 @@ from typing import Dict, List
 
 import torch
 
-from ..models.configs import (ChunkAttnSpec, DeltaSpec, LatentAttnSpec, LayerSpec, ModelConfig, MoESpec, SSDSpec,
-                              WindowAttnSpec, PRESETS)
+from ..models.configs import (ChunkAttnSpec, DeltaSpec, GatedAttnSpec, LatentAttnSpec, LayerSpec, ModelConfig, MoESpec,
+                              SSDSpec, WindowAttnSpec, PRESETS)
 from ..models.decoder import build_model
 from ..models.hybrid import build_hybrid
 from .generate import Generator, SamplingParams
@@ -113,6 +117,39 @@ def vetevik_config(s: dict) -> ModelConfig:
                        residual_mult=0.3)
 
 
+# Fikupel sizes: latent-attention and gated-attention layers alternate; width, head count, head sizes, window
+# (= Vetevik's chunk) and experts as in the Vetevik size of the same name, latent ranks as in the Pagonex one;
+# the first layer's PolyNorm feed-forward is as wide as the experts' active width
+FIKUPEL_SIZES = {
+    "w1024": dict(width=1024, layers=4, heads=16, kv=4, dim=64, window=512, keep=4, rot=32, q_rank=384, kv_rank=128,
+                  experts=16, top=4, ff=1024, dense_ff=4096, streams=2, vocab=32000),
+    "w2048": dict(width=2048, layers=4, heads=16, kv=4, dim=128, window=1024, keep=4, rot=64, q_rank=768, kv_rank=256,
+                  experts=32, top=4, ff=2048, dense_ff=8192, streams=2, vocab=32000),
+}
+
+
+def fikupel_config(s: dict) -> ModelConfig:
+    moe = MoESpec(s["experts"], s["top"], 1.0, s["ff"], router="top_softmax", act="silu_glu", weight_on="output",
+                  router_bias=True)
+    llama3 = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+              "original_max_position_embeddings": 8192.0}
+    specs = []
+    for i in range(s["layers"]):
+        ff = dict(ff=s["dense_ff"], ff_act="polynorm") if i == 0 else dict(moe=moe, ff_act="polynorm")
+        if i % 2 == 0:
+            a = LatentAttnSpec(s["heads"], s["dim"], 0, s["dim"], s["q_rank"], s["kv_rank"], s["dim"] ** -0.5, s["window"],
+                               sink=True)
+            specs.append(LayerSpec("latent_attention", latent=a, **ff))
+        else:
+            a = GatedAttnSpec(s["heads"], s["kv"], s["dim"], s["dim"], s["dim"] ** -0.5, s["window"], s["keep"], s["rot"],
+                              500000.0, llama3)
+            specs.append(LayerSpec("gated_attention", gated_attn=a, **ff))
+    return ModelConfig(arch="fikupel", vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
+                       num_heads=s["heads"], num_kv_heads=s["kv"], intermediate_size=0, head_dim=s["dim"],
+                       max_position_embeddings=1 << 20, norm="rms", norm_eps=1e-6, act="silu_glu", pos_emb="rope",
+                       tie_word_embeddings=True, name="fikupel-bench", layer_specs=specs, streams=s["streams"], hyper=True)
+
+
 def closest_config(s: dict) -> ModelConfig:
     return PRESETS["phi-2"].replace(vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
                                     num_heads=s["heads"], num_kv_heads=s["kv"], head_dim=s["dim"], rotary_dim=s["dim"],
@@ -162,7 +199,8 @@ def op_times(eng: RaggedEngine, entries, close=()) -> Dict[str, float]:
              "rope_paged_write", "pool_blocks", "window_pool_attention", "conv_silu", "ssd_scan", "linear_f32",
              "embedding_bigram", "canon_conv", "layer_norm_rows", "layer_norm_residual", "rms_norm_cols", "glu_clamp",
              "latent_write", "delta_prepare", "delta_rule_scan", "head_norm_gate", "moe_route", "moe_experts",
-             "group_rms_norm", "group_norm_residual", "chunk_attention", "delta_prepare_head"]
+             "group_rms_norm", "group_norm_residual", "chunk_attention", "delta_prepare_head", "glu_silu",
+             "hyper_read_norm", "hyper_update", "poly_norm", "qk_norm_rope_write", "unrotate_gate"]
     saved = {n: getattr(seqmix, n) for n in names}
     lin = F.linear
 
@@ -256,12 +294,31 @@ def run_vetevik(sizes: List[str], prompt: int, batch: int, steps: int, device) -
             "decode_batch": batch, "decode_steps": steps, "sizes": res}
 
 
+def run_fikupel(sizes: List[str], prompt: int, batch: int, steps: int, device) -> Dict:
+    res = {}
+    r2 = lambda d: {k: (round(v, 2) if isinstance(v, float) else v) for k, v in d.items()}
+    for name in sizes:
+        s, c = FIKUPEL_SIZES[name], VETEVIK_SIZES[name]
+        f = bench_hybrid(s, prompt, batch, steps, device, fikupel_config(s))
+        torch.cuda.empty_cache()
+        v = bench_hybrid(c, prompt, batch, steps, device, vetevik_config(c))
+        torch.cuda.empty_cache()
+        res[name] = {"size": s, "closest_size": c, "fikupel": r2(f), "closest_vetevik": r2(v),
+                     "prefill_ratio": round(f["prefill_tok_s"] / v["prefill_tok_s"], 3),
+                     "decode_ratio": round(f["decode_tok_s"] / v["decode_tok_s"], 3)}
+    return {"metric": "prefill / decode tokens/s, Fikupel layer-spec model vs the Vetevik model of equal size",
+            "dtype": "bf16", "data": "synthetic (random weights, random prompt)", "prompt_tokens": prompt,
+            "decode_batch": batch, "decode_steps": steps, "sizes": res}
+
+
 def run(sizes: List[str], prompt: int = 4096, batch: int = 4, steps: int = 32, device=None, family: str = "nudadra") -> Dict:
     device = torch.device(device or "cuda:0")
     if family == "pagonex":
         return run_pagonex(sizes, prompt, batch, steps, device)
     if family == "vetevik":
         return run_vetevik(sizes, prompt, batch, steps, device)
+    if family == "fikupel":
+        return run_fikupel(sizes, prompt, batch, steps, device)
     res = {}
     for name in sizes:
         s = SIZES[name]

@@ -649,7 +649,7 @@ def test_graph_replays_against_eager_steps(tmp_path):
     the replays, against the same schedule stepped eagerly."""
     cfg = CONFIGS["two_streams"]()
     w = make_weights(cfg, 19)
-    reqs = {"a": tokens(40, cfg["vocab"], 1), "b": tokens(33, cfg["vocab"], 2)}
+    reqs = {"a": tokens(40, cfg["vocab"], 1), "b": tokens(32, cfg["vocab"], 2)}
     sched = [[("a", 20), ("b", 9)]] + [[("a", 1), ("b", 1)]] * 8 + [[("a", 4), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 8 + \
         [[("b", 6)]]
     model = load(tmp_path, cfg, w, "cuda")
