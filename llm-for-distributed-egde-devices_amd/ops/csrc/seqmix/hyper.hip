@@ -56,7 +56,8 @@ __global__ void __launch_bounds__(NT) hyper_read_norm_kernel(const float* __rest
 
 // X [rows, S, W] fp32 in place: X[t, r] <- sum_s mix[s, r] X[t, s] + out_w[r] v, v = y[t] + sum_k pw[t, k] parts[t, k]
 // (fp32, k order; y / parts / pw may be null; pw null with parts: ones).  mix null: X[t, r] += v.
-template <typename T>
+// C = columns per thread and pass (4 with 16-byte stream accesses when W % 4 == 0, else 1).
+template <typename T, int C>
 __global__ void __launch_bounds__(NT) hyper_update_kernel(float* __restrict__ X, const float* __restrict__ mix,
                                                           const float* __restrict__ out_w, const T* __restrict__ y,
                                                           const T* __restrict__ parts, const float* __restrict__ pw, int K,
@@ -68,57 +69,118 @@ __global__ void __launch_bounds__(NT) hyper_update_kernel(float* __restrict__ X,
     __syncthreads();
   }
   float* xr = X + t * S * W;
-  for (int c = blockIdx.y * NT + threadIdx.x; c < W; c += gridDim.y * NT) {
-    float v = y ? ldf<T>(y + t * W + c) : 0.f;
-    for (int k = 0; k < K; ++k) {
-      const float p = ldf<T>(parts + (t * K + k) * W + c);
-      v += pw ? pw[t * K + k] * p : p;
+  auto ld4 = [&](const T* p, float* f) {                     // C consecutive activations
+    if constexpr (C == 1) f[0] = ldf<T>(p);
+    else if constexpr (sizeof(T) == 4) {
+      const float4 a = *reinterpret_cast<const float4*>(p);
+      f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
+    } else {
+      const uint2 a = *reinterpret_cast<const uint2*>(p);
+      f[0] = __uint_as_float(a.x << 16); f[1] = __uint_as_float(a.x & 0xffff0000u);
+      f[2] = __uint_as_float(a.y << 16); f[3] = __uint_as_float(a.y & 0xffff0000u);
     }
-    float xs[MAXS];
+  };
+  for (int c = (blockIdx.y * NT + threadIdx.x) * C; c < W; c += gridDim.y * NT * C) {
+    float v[C];
 #pragma unroll
-    for (int s = 0; s < MAXS; ++s) xs[s] = s < S ? xr[(size_t)s * W + c] : 0.f;
+    for (int i = 0; i < C; ++i) v[i] = 0.f;
+    if (y) ld4(y + t * W + c, v);
+    for (int k = 0; k < K; ++k) {
+      float p[C];
+      ld4(parts + (t * K + k) * W + c, p);
+      const float wk = pw ? pw[t * K + k] : 1.f;
+#pragma unroll
+      for (int i = 0; i < C; ++i) v[i] += wk * p[i];
+    }
+    float xs[MAXS][C];
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+      if (s < S) {
+        if constexpr (C == 4) {
+          const float4 a = *reinterpret_cast<const float4*>(xr + (size_t)s * W + c);
+          xs[s][0] = a.x; xs[s][1] = a.y; xs[s][2] = a.z; xs[s][3] = a.w;
+        } else {
+          xs[s][0] = xr[(size_t)s * W + c];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < C; ++i) xs[s][i] = 0.f;
+      }
+    }
 #pragma unroll
     for (int r = 0; r < MAXS; ++r) {
       if (r < S) {
-        float n;
-        if (mix) {
-          n = 0.f;
+        float n[C];
 #pragma unroll
-          for (int s = 0; s < MAXS; ++s)
-            if (s < S) n += m_s[s * S + r] * xs[s];
-          n += m_s[S * S + r] * v;
-        } else {
-          n = xs[r] + v;
+        for (int i = 0; i < C; ++i) {
+          if (mix) {
+            float a = 0.f;
+#pragma unroll
+            for (int s = 0; s < MAXS; ++s)
+              if (s < S) a += m_s[s * S + r] * xs[s][i];
+            n[i] = a + m_s[S * S + r] * v[i];
+          } else {
+            n[i] = xs[r][i] + v[i];
+          }
         }
-        xr[(size_t)r * W + c] = n;
+        if constexpr (C == 4) *reinterpret_cast<float4*>(xr + (size_t)r * W + c) = make_float4(n[0], n[1], n[2], n[3]);
+        else xr[(size_t)r * W + c] = n[0];
       }
     }
   }
 }
 
 // z [rows, F] -> a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row.  LDS: z [F] fp32.
-template <typename T>
+// VEC (F, ld % 8 == 0, 32-byte aligned rows): 8 coordinates per thread and pass.
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) poly_norm_kernel(const T* __restrict__ z, int ld, const float* __restrict__ coef,
                                                        T* __restrict__ y, int F, float eps) {
   extern __shared__ __attribute__((aligned(16))) float z_s[];
   __shared__ float red[NT / 64];
   const size_t t = blockIdx.x;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-  for (int c = threadIdx.x; c < F; c += NT) {
-    const float v = ldf<T>(z + t * ld + c), v2 = v * v;
-    z_s[c] = v;
-    s2 += v2;
-    s4 += v2 * v2;
-    s6 += v2 * v2 * v2;
+  if constexpr (VEC) {
+    for (int c = threadIdx.x * 8; c < F; c += NT * 8) {
+      float v[8];
+      load8<T>(z + t * ld + c, v);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float v2 = v[i] * v[i];
+        z_s[c + i] = v[i];
+        s2 += v2;
+        s4 += v2 * v2;
+        s6 += v2 * v2 * v2;
+      }
+    }
+  } else {
+    for (int c = threadIdx.x; c < F; c += NT) {
+      const float v = ldf<T>(z + t * ld + c), v2 = v * v;
+      z_s[c] = v;
+      s2 += v2;
+      s4 += v2 * v2;
+      s6 += v2 * v2 * v2;
+    }
   }
   const float inv = 1.f / (float)F;
   const float r1 = coef[0] / sqrtf(block_sum<NT>(s2, red) * inv + eps);
   const float r2 = coef[1] / sqrtf(block_sum<NT>(s4, red) * inv + eps);
   const float r3 = coef[2] / sqrtf(block_sum<NT>(s6, red) * inv + eps);
   const float e = coef[3];
-  for (int c = threadIdx.x; c < F; c += NT) {
-    const float v = z_s[c];
-    stf<T>(y + t * F + c, v * r1 + v * v * r2 + v * v * v * r3 + e);
+  if constexpr (VEC) {
+    for (int c = threadIdx.x * 8; c < F; c += NT * 8) {      // every thread reads back the chunk it wrote
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float v = z_s[c + i];
+        o[i] = v * r1 + v * v * r2 + v * v * v * r3 + e;
+      }
+      store8<T>(y + t * F + c, o);
+    }
+  } else {
+    for (int c = threadIdx.x; c < F; c += NT) {
+      const float v = z_s[c];
+      stf<T>(y + t * F + c, v * r1 + v * v * r2 + v * v * v * r3 + e);
+    }
   }
 }
 
@@ -177,6 +239,67 @@ __global__ void __launch_bounds__(NT) qk_norm_rope_write_kernel(
   }
 }
 
+// The same with 8 coordinates per thread (D, Dv, ld % 8 == 0, 32-byte aligned rows): a head (q, k or v) is held
+// by LPH = max(D, Dv) / 8 neighbouring threads, NT / LPH heads per workgroup (blockIdx.y walks the rest); one 16- /
+// 32-byte load per thread, the head's sum of squares from the threads' shares through LDS, then norm, turn (a
+// rotation pair never leaves its chunk), temperature and one 16- / 32-byte store.
+template <typename T>
+__global__ void __launch_bounds__(NT) qk_norm_rope_write_vec_kernel(
+    const T* __restrict__ proj, int ld, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+    const int* __restrict__ seq_slot, const int* __restrict__ ptab, int ptab_ld, const float* __restrict__ qw,
+    const float* __restrict__ kw, float eps, const float* __restrict__ cs, const float* __restrict__ vcs,
+    const float* __restrict__ temp, T* __restrict__ q_out, T* __restrict__ kp, T* __restrict__ vp, int H, int G, int D,
+    int Dv, int rot, int page, int LPH) {
+  __shared__ float part_s[NT];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int unit = blockIdx.y * (NT / LPH) + tid / LPH, d = (tid % LPH) * 8;
+  const bool isv = unit >= H + G, isq = unit < H;
+  const int size = isv ? Dv : D;
+  const bool live = tid / LPH < NT / LPH && unit < H + 2 * G && d < size;
+  const float* w = isv ? nullptr : (isq ? qw : kw);
+  float v[8];
+  float ss = 0.f;
+  if (live) {
+    load8<T>(proj + (size_t)t * ld + (isv ? (size_t)(H + G) * D + (size_t)(unit - H - G) * Dv : (size_t)unit * D) + d, v);
+    if (w) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+    }
+  }
+  part_s[tid] = ss;
+  __syncthreads();
+  if (!live) return;
+  const int pos = tok_pos[t], slot = seq_slot[tok_seq[t]];
+  const size_t prow = (size_t)ptab[(size_t)slot * ptab_ld + pos / page] * page + pos % page;
+  if (w) {
+    float tot = 0.f;
+    const int first = (tid / LPH) * LPH;
+    for (int i = 0; i < D / 8; ++i) tot += part_s[first + i];
+    const float r = 1.f / sqrtf(tot / (float)D + eps);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] *= r * w[d + i];
+  }
+  const float* c = isv ? (vcs ? vcs + (size_t)pos * Dv : nullptr) : ((cs && d < rot) ? cs + (size_t)pos * rot : nullptr);
+  if (c) {
+    const int lim = isv ? Dv : rot;
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      if (d + i < lim) {
+        const float co = c[d + i], si = c[d + i + 1], a = v[i], b = v[i + 1];
+        v[i] = a * co - b * si;
+        v[i + 1] = b * co + a * si;
+      }
+    }
+  }
+  if (isq && temp) {
+    const float mul = temp[unit];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] *= mul;
+  }
+  T* dst = isq ? q_out + ((size_t)t * H + unit) * D : isv ? vp + (prow * G + (unit - H - G)) * Dv : kp + (prow * G + (unit - H)) * D;
+  store8<T>(dst + d, v);
+}
+
 // a [rows, H * Dv]: every head's pairs (2m, 2m + 1) turned by -pos (vcs[pos, m] = (cos, sin); null: as it is), then
 // times sigmoid(gate[t, e]) (null: 1).
 template <typename T>
@@ -225,9 +348,15 @@ int edge_sm_hyper_update(float* X, const float* mix, const float* out_w, const v
                          int K, int rows, int S, int W, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   if (S < 1 || S > MAXS || (!y && K == 0) || (mix && !out_w)) return -2;
-  const int gy = rows >= 1024 ? 1 : (W + NT - 1) / NT < 8 ? (W + NT - 1) / NT : 8;
-  SM_T(f32, hipLaunchKernelGGL(hyper_update_kernel<T>, dim3(rows, gy), dim3(NT), 0, st, X, mix, out_w, (const T*)y,
-                               (const T*)parts, pw, K, S, W));
+  const bool vec = W % 4 == 0 && (((uintptr_t)X | (uintptr_t)y | (uintptr_t)parts) & 15) == 0;
+  const int per = NT * (vec ? 4 : 1);
+  const int gy = rows >= 1024 ? 1 : (W + per - 1) / per < 8 ? (W + per - 1) / per : 8;
+  if (vec)
+    SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 4>), dim3(rows, gy), dim3(NT), 0, st, X, mix, out_w, (const T*)y,
+                                 (const T*)parts, pw, K, S, W));
+  else
+    SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 1>), dim3(rows, gy), dim3(NT), 0, st, X, mix, out_w, (const T*)y,
+                                 (const T*)parts, pw, K, S, W));
   return (int)hipGetLastError();
 }
 
@@ -235,8 +364,12 @@ int edge_sm_poly_norm(const void* z, int ld, const float* coef, void* y, int row
                       hipStream_t st) {
   if (rows == 0 || F == 0) return 0;
   if ((size_t)F * 4 > 60 * 1024) return -3;
-  SM_T(f32, hipLaunchKernelGGL(poly_norm_kernel<T>, dim3(rows), dim3(NT), (size_t)F * 4, st, (const T*)z, ld, coef, (T*)y,
-                               F, eps));
+  if (F % 8 == 0 && ld % 8 == 0 && (((uintptr_t)z | (uintptr_t)y) & 31) == 0)
+    SM_T(f32, hipLaunchKernelGGL((poly_norm_kernel<T, true>), dim3(rows), dim3(NT), (size_t)F * 4, st, (const T*)z, ld, coef,
+                                 (T*)y, F, eps));
+  else
+    SM_T(f32, hipLaunchKernelGGL((poly_norm_kernel<T, false>), dim3(rows), dim3(NT), (size_t)F * 4, st, (const T*)z, ld, coef,
+                                 (T*)y, F, eps));
   return (int)hipGetLastError();
 }
 
@@ -246,9 +379,16 @@ int edge_sm_qk_norm_rope_write(const void* proj, int ld, const int* tok_seq, con
                                int D, int Dv, int rot, int page, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   if (rot % 2 || rot > D || (rot > 0 && !cs) || (vcs && Dv % 2)) return -2;
-  SM_T(f32, hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(rows), dim3(NT), 0, st, (const T*)proj, ld, tok_seq,
-                               tok_pos, seq_slot, ptab, ptab_ld, qw, kw, eps, rot > 0 ? cs : nullptr, vcs, temp, (T*)q_out,
-                               (T*)kp, (T*)vp, H, G, D, Dv, rot, page));
+  const int lph = (D > Dv ? D : Dv) / 8;                      // threads per head
+  if (D % 8 == 0 && Dv % 8 == 0 && ld % 8 == 0 && lph >= 1 && lph <= NT &&
+      (((uintptr_t)proj | (uintptr_t)q_out | (uintptr_t)kp | (uintptr_t)vp) & 31) == 0)
+    SM_T(f32, hipLaunchKernelGGL(qk_norm_rope_write_vec_kernel<T>, dim3(rows, (H + 2 * G + NT / lph - 1) / (NT / lph)), dim3(NT),
+                                 0, st, (const T*)proj, ld, tok_seq, tok_pos, seq_slot, ptab, ptab_ld, qw, kw, eps,
+                                 rot > 0 ? cs : nullptr, vcs, temp, (T*)q_out, (T*)kp, (T*)vp, H, G, D, Dv, rot, page, lph));
+  else
+    SM_T(f32, hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(rows), dim3(NT), 0, st, (const T*)proj, ld, tok_seq,
+                                 tok_pos, seq_slot, ptab, ptab_ld, qw, kw, eps, rot > 0 ? cs : nullptr, vcs, temp, (T*)q_out,
+                                 (T*)kp, (T*)vp, H, G, D, Dv, rot, page));
   return (int)hipGetLastError();
 }
 
