@@ -762,3 +762,65 @@ def test_sizes_that_are_not_multiples_of_eight(tmp_path, precision):
         assert e.max().item() < TOL["fp32"]
     else:
         assert e.median().item() < 3e-2 and e.quantile(0.9).item() < 0.1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,T", [(16, 4, 16400), (12, 6, 11100)])
+def test_prompt_attention_with_grouped_heads_on_long_prompts(H, G, T):
+    """Prompts long enough that the matrix-core kernel serves four (or two) query heads of a kv head from one
+    staged tile, with window, kept tokens and sink over separate key and value pages: against the general fp32
+    kernel on the same bf16-rounded inputs (which the oracle pins)."""
+    D, Dv, window, keep = 64, 64, 200, 70
+    g = torch.Generator().manual_seed(1)
+    q = (torch.randn(T, H, D, generator=g) * 0.7).to(torch.bfloat16)
+    k, v = torch.randn(T, G, D, generator=g).to(torch.bfloat16), torch.randn(T, G, Dv, generator=g).to(torch.bfloat16)
+    sink = torch.randn(H, generator=g).cuda()
+    spec = _Spec(kv_heads=G, dim=D, vdim=Dv)
+    outs = []
+    for dt in (torch.float32, torch.bfloat16):
+        cache = PagedCache([_Spec(latent=None, delta=None, moe=None, attn=None, ssd=None, chunk_attn=None, gated_attn=spec)],
+                           (T + 63) // 64, slots=1, page=64, dtype=dt, device="cuda")
+        run, slot = cache.run(0), cache.acquire()
+        cache.extend(slot, T)
+        meta = seqmix.RaggedMeta.build([(slot, 0, T)], cache.page_table, cache.page, "cuda")
+        pos = torch.arange(T, device="cuda")
+        pid = cache.page_table[slot, pos // 64].long()
+        run.k[pid, pos % 64], run.v[pid, pos % 64] = k.cuda().to(dt), v.cuda().to(dt)
+        outs.append(seqmix.window_pool_attention(q.cuda().to(dt), None, run.k, run.v, None, None, meta, D ** -0.5, window, None,
+                                                 sink, keep).float().cpu())
+    assert (outs[0] - outs[1]).abs().max() < 0.05
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,Dv,rot", [(16, 4, 128, 128, 64), (32, 8, 96, 64, 96), (5, 5, 40, 72, 8), (64, 8, 64, 128, 0),
+                                          (3, 1, 7, 10, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_rotation_and_cache_write_at_many_head_shapes(H, G, D, Dv, rot, dtype):
+    """The q / k norm + rotation + temperature + rotated-value write and the turn back + gate kernels against their
+    PyTorch forms on the same inputs: heads spread over several workgroups, head sizes whose thread groups do
+    not divide a workgroup, the scalar forms at odd sizes."""
+    from edgellm import ops
+    g = torch.Generator().manual_seed(H + D)
+    T, extra = 37, 8
+    proj = torch.randn(T, (H + G) * D + G * Dv + extra, generator=g).to(dtype)
+    qw, kw, temp = (1 + 0.2 * torch.randn(D, generator=g)), (1 + 0.2 * torch.randn(D, generator=g)), 0.5 + torch.rand(H, generator=g)
+    rope = ops.rope_tables(rot, 256, 100.0, None) if rot else None
+    vrope = ops.rope_tables(Dv, 256, 100.0, None)
+    spec = _Spec(kv_heads=G, dim=D, vdim=Dv)
+    res = {}
+    for dev in ("cpu", "cuda"):
+        cache = PagedCache([_Spec(latent=None, delta=None, moe=None, attn=None, ssd=None, chunk_attn=None, gated_attn=spec)], 4,
+                           slots=2, page=64, dtype=dtype, device=dev)
+        run = cache.run(0)
+        s0, s1 = cache.acquire(), cache.acquire()
+        cache.extend(s0, 90), cache.extend(s1, 100)
+        meta = seqmix.RaggedMeta.build([(s0, 60, 30), (s1, 93, 7)], cache.page_table, cache.page, dev)
+        D_ = lambda t: None if t is None else t.to(dev)
+        q = seqmix.qk_norm_rope_write(D_(proj), meta, D_(qw), D_(kw), 1e-5, D_(rope), D_(vrope), D_(temp), run.k, run.v, H, rot)
+        a = torch.randn(T, H * Dv, generator=torch.Generator().manual_seed(3)).to(dtype)
+        gate = torch.randn(T, H * Dv + 3, generator=torch.Generator().manual_seed(4)).to(dtype)
+        o = seqmix.unrotate_gate(D_(a), D_(gate)[:, 3:], meta, D_(vrope), H)
+        res[dev] = [t.float().cpu() for t in (q, run.k, run.v, o)]
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for c, d in zip(res["cpu"], res["cuda"]):
+        assert torch.allclose(c, d, atol=tol, rtol=tol)
