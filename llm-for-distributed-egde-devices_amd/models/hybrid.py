@@ -202,20 +202,37 @@ class HyperLayer(nn.Module):
             self.norm2 = StreamNorm(W, eps, device)
             self.hc2 = HyperConnection(cfg.streams, device) if cfg.hyper else None
 
-    def forward(self, X: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+    def first_read(self) -> tuple:
+        """(read weights, norm weight, eps) of the mixer's input: the layer before computes it while it rebuilds
+        the streams."""
+        return (self.hc1.inp if self.hc1 is not None else None, self.norm1.weight, self.norm1.eps)
+
+    def forward(self, X: torch.Tensor, meta: seqmix.RaggedMeta, run, h: Optional[torch.Tensor] = None,
+                nxt: Optional[tuple] = None):
+        """``h``: this layer's first input when the layer before already computed it; ``nxt``: the next layer's
+        ``first_read()``.  Returns (X, the next layer's first input or None).  Every rebuild of the streams but
+        the model's last also reads and norms them for the sublayer that follows, in the same kernel."""
         hc = self.hc1
-        y = self.mix(self.norm1(X, hc.inp if hc is not None else None, self.dtype), meta, run)
-        seqmix.hyper_update(X, hc.mix if hc is not None else None, hc.out if hc is not None else None, y)
-        if self.ff is not None:
-            hc = self.hc2
-            h = self.norm2(X, hc.inp if hc is not None else None, self.dtype)
-            mix, out = (hc.mix, hc.out) if hc is not None else (None, None)
-            if self.spec.moe is not None:
-                shared, parts, wts = self.ff(h)
-                seqmix.hyper_update(X, mix, out, shared, parts, wts)
-            else:
-                seqmix.hyper_update(X, mix, out, self.ff(h))
-        return X
+        if h is None:
+            h = self.norm1(X, hc.inp if hc is not None else None, self.dtype)
+        y = self.mix(h, meta, run)
+        mix, out = (hc.mix, hc.out) if hc is not None else (None, None)
+        if self.ff is None:
+            if nxt is not None:
+                return X, seqmix.hyper_update(X, mix, out, y, nxt=nxt)
+            seqmix.hyper_update(X, mix, out, y)
+            return X, None
+        hc = self.hc2
+        h = seqmix.hyper_update(X, mix, out, y, nxt=(hc.inp if hc is not None else None, self.norm2.weight, self.norm2.eps))
+        mix, out = (hc.mix, hc.out) if hc is not None else (None, None)
+        if self.spec.moe is not None:
+            shared, parts, wts = self.ff(h)
+        else:
+            shared, parts, wts = self.ff(h), None, None
+        if nxt is not None:
+            return X, seqmix.hyper_update(X, mix, out, shared, parts, wts, nxt=nxt)
+        seqmix.hyper_update(X, mix, out, shared, parts, wts)
+        return X, None
 
 
 def _make_layer(cfg: ModelConfig, spec: LayerSpec, idx: int, dtype, device) -> nn.Module:
@@ -288,6 +305,7 @@ class HybridLM(nn.Module):
         x = x0.clone() if cfg.loop is not None else x0
         if cfg.streams:                                  # [T, S, W]: every stream starts as the embedding rows
             x = x0[:, None, :].expand(-1, cfg.streams, -1).contiguous()
+        h_next = None
         for r, (i, t) in enumerate(self.runs):
             if t is not None and i == cfg.loop.start:
                 if cfg.loop.entry == "add_embed":
@@ -295,7 +313,11 @@ class HybridLM(nn.Module):
                         x.add_(x0)
                 else:
                     x = seqmix.linear_f32(seqmix.cat_cast(x, x0, self.dtype), self.loop_in.weight, self.loop_step[t])
-            x = self.layers[i](x, meta, cache.run(r))
+            if cfg.streams:                              # the next layer's read + norm rides on this layer's last rebuild
+                nxt = self.layers[self.runs[r + 1][0]].first_read() if r + 1 < len(self.runs) and cfg.loop is None else None
+                x, h_next = self.layers[i](x, meta, cache.run(r), h_next, nxt)
+            else:
+                x = self.layers[i](x, meta, cache.run(r))
             if taps is not None:
                 taps.append(x.sum(1) if cfg.streams else x.clone())
         if rows is not None:

@@ -84,7 +84,8 @@ int edge_sm_moe_route(const void* h, int W, const float* router, const float* bi
 int edge_sm_hyper_read_norm(const float* X, const float* in_w, const float* w, void* y, int rows, int S, int W, float eps,
                             int f32, hipStream_t st);
 int edge_sm_hyper_update(float* X, const float* mix, const float* out_w, const void* y, const void* parts, const float* pw,
-                         int K, int rows, int S, int W, int f32, hipStream_t st);
+                         int K, int rows, int S, int W, const float* in2, const float* w2, void* h, float eps, int f32,
+                         hipStream_t st);
 int edge_sm_poly_norm(const void* z, int ld, const float* coef, void* y, int rows, int F, float eps, int f32,
                       hipStream_t st);
 int edge_sm_qk_norm_rope_write(const void* proj, int ld, const int* tok_seq, const int* tok_pos, const int* seq_slot,
@@ -773,9 +774,12 @@ at::Tensor sm_hyper_read_norm(const at::Tensor& X, const std::optional<at::Tenso
   return y;
 }
 
-void sm_hyper_update(at::Tensor& X, const std::optional<at::Tensor>& mix, const std::optional<at::Tensor>& out_w,
-                     const std::optional<at::Tensor>& y, const std::optional<at::Tensor>& parts,
-                     const std::optional<at::Tensor>& part_w) {
+// next_w given: also returns the next sublayer's input, norm(sum_r next_in[r] X_new[:, r]) next_w, in the dtype of y / parts
+std::optional<at::Tensor> sm_hyper_update(at::Tensor& X, const std::optional<at::Tensor>& mix,
+                                          const std::optional<at::Tensor>& out_w, const std::optional<at::Tensor>& y,
+                                          const std::optional<at::Tensor>& parts, const std::optional<at::Tensor>& part_w,
+                                          const std::optional<at::Tensor>& next_in, const std::optional<at::Tensor>& next_w,
+                                          double eps) {
   chk_f32(X, "X");
   TORCH_CHECK(X.dim() == 3 && (y || parts) && bool(mix) == bool(out_w), "X fp32 [T, S, W]; y or parts; mix with out_w");
   const int64_t T = X.size(0), S = X.size(1), W = X.size(2);
@@ -801,10 +805,23 @@ void sm_hyper_update(at::Tensor& X, const std::optional<at::Tensor>& mix, const 
     }
   }
   c10::hip::HIPGuardMasqueradingAsCUDA guard(X.device());
+  std::optional<at::Tensor> h;
+  if (next_w) {
+    chk_f32(*next_w, "next_w");
+    TORCH_CHECK(next_w->numel() == W, "next_w: fp32 [W]");
+    if (next_in) {
+      chk_f32(*next_in, "next_in");
+      TORCH_CHECK(next_in->numel() == S, "next_in: fp32 [S]");
+    }
+    h = at::empty({T, W}, X.options().dtype(act_type(is_f32)));
+  }
   check(edge_sm_hyper_update(X.data_ptr<float>(), mix ? mix->data_ptr<float>() : nullptr,
                              out_w ? out_w->data_ptr<float>() : nullptr, y ? y->data_ptr() : nullptr,
                              parts ? parts->data_ptr() : nullptr, parts && part_w ? part_w->data_ptr<float>() : nullptr, K,
-                             (int)T, (int)S, (int)W, is_f32, stream()), "sm_hyper_update");
+                             (int)T, (int)S, (int)W, (h && next_in) ? next_in->data_ptr<float>() : nullptr,
+                             h ? next_w->data_ptr<float>() : nullptr, h ? h->data_ptr() : nullptr, (float)eps, is_f32,
+                             stream()), "sm_hyper_update");
+  return h;
 }
 
 at::Tensor sm_poly_norm(const at::Tensor& z, const at::Tensor& coef, double eps) {

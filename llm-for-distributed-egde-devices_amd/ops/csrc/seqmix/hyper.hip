@@ -57,13 +57,22 @@ __global__ void __launch_bounds__(NT) hyper_read_norm_kernel(const float* __rest
 // X [rows, S, W] fp32 in place: X[t, r] <- sum_s mix[s, r] X[t, s] + out_w[r] v, v = y[t] + sum_k pw[t, k] parts[t, k]
 // (fp32, k order; y / parts / pw may be null; pw null with parts: ones).  mix null: X[t, r] += v.
 // C = columns per thread and pass (4 with 16-byte stream accesses when W % 4 == 0, else 1).
-template <typename T, int C>
+// NEXT: the next sublayer's read and norm in the same pass (one workgroup per token, dynamic LDS u [W]):
+// h[t] = u / sqrt(mean(u^2) + eps) * w2 with u = sum_r in2[r] X_new[t, r] (in2 null: the plain sum).
+template <typename T, int C, bool NEXT>
 __global__ void __launch_bounds__(NT) hyper_update_kernel(float* __restrict__ X, const float* __restrict__ mix,
                                                           const float* __restrict__ out_w, const T* __restrict__ y,
                                                           const T* __restrict__ parts, const float* __restrict__ pw, int K,
-                                                          int S, int W) {
+                                                          int S, int W, const float* __restrict__ in2,
+                                                          const float* __restrict__ w2, T* __restrict__ h, float eps) {
+  extern __shared__ __attribute__((aligned(16))) float u_s[];
   __shared__ float m_s[MAXS * MAXS + MAXS];
+  __shared__ float red[NT / 64];
   const size_t t = blockIdx.x;
+  float a2[MAXS];
+  float ss = 0.f;
+#pragma unroll
+  for (int s = 0; s < MAXS; ++s) a2[s] = (NEXT && s < S) ? (in2 ? in2[s] : 1.f) : 0.f;
   if (mix) {
     for (int e = threadIdx.x; e < S * S + S; e += NT) m_s[e] = e < S * S ? mix[e] : out_w[e - S * S];
     __syncthreads();
@@ -107,6 +116,9 @@ __global__ void __launch_bounds__(NT) hyper_update_kernel(float* __restrict__ X,
         for (int i = 0; i < C; ++i) xs[s][i] = 0.f;
       }
     }
+    float u[C];
+#pragma unroll
+    for (int i = 0; i < C; ++i) u[i] = 0.f;
 #pragma unroll
     for (int r = 0; r < MAXS; ++r) {
       if (r < S) {
@@ -122,11 +134,20 @@ __global__ void __launch_bounds__(NT) hyper_update_kernel(float* __restrict__ X,
           } else {
             n[i] = xs[r][i] + v[i];
           }
+          if constexpr (NEXT) u[i] += a2[r] * n[i];
         }
         if constexpr (C == 4) *reinterpret_cast<float4*>(xr + (size_t)r * W + c) = make_float4(n[0], n[1], n[2], n[3]);
         else xr[(size_t)r * W + c] = n[0];
       }
     }
+    if constexpr (NEXT) {
+#pragma unroll
+      for (int i = 0; i < C; ++i) { u_s[c + i] = u[i]; ss += u[i] * u[i]; }
+    }
+  }
+  if constexpr (NEXT) {
+    const float r = 1.f / sqrtf(block_sum<NT>(ss, red) / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += NT) stf<T>(h + t * W + c, u_s[c] * r * w2[c]);
   }
 }
 
@@ -344,19 +365,31 @@ int edge_sm_hyper_read_norm(const float* X, const float* in_w, const float* w, v
   return (int)hipGetLastError();
 }
 
+// w2 given: the next sublayer's input h [rows, W] = norm(sum_r in2[r] X_new[:, r]) w2 is written in the same pass
 int edge_sm_hyper_update(float* X, const float* mix, const float* out_w, const void* y, const void* parts, const float* pw,
-                         int K, int rows, int S, int W, int f32, hipStream_t st) {
+                         int K, int rows, int S, int W, const float* in2, const float* w2, void* h, float eps, int f32,
+                         hipStream_t st) {
   if (rows == 0) return 0;
-  if (S < 1 || S > MAXS || (!y && K == 0) || (mix && !out_w)) return -2;
+  if (S < 1 || S > MAXS || (!y && K == 0) || (mix && !out_w) || (w2 && !h)) return -2;
   const bool vec = W % 4 == 0 && (((uintptr_t)X | (uintptr_t)y | (uintptr_t)parts) & 15) == 0;
+  if (w2) {
+    if ((size_t)W * 4 > 60 * 1024) return -3;
+    if (vec)
+      SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 4, true>), dim3(rows), dim3(NT), (size_t)W * 4, st, X, mix, out_w,
+                                   (const T*)y, (const T*)parts, pw, K, S, W, in2, w2, (T*)h, eps));
+    else
+      SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 1, true>), dim3(rows), dim3(NT), (size_t)W * 4, st, X, mix, out_w,
+                                   (const T*)y, (const T*)parts, pw, K, S, W, in2, w2, (T*)h, eps));
+    return (int)hipGetLastError();
+  }
   const int per = NT * (vec ? 4 : 1);
   const int gy = rows >= 1024 ? 1 : (W + per - 1) / per < 8 ? (W + per - 1) / per : 8;
   if (vec)
-    SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 4>), dim3(rows, gy), dim3(NT), 0, st, X, mix, out_w, (const T*)y,
-                                 (const T*)parts, pw, K, S, W));
+    SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 4, false>), dim3(rows, gy), dim3(NT), 0, st, X, mix, out_w,
+                                 (const T*)y, (const T*)parts, pw, K, S, W, nullptr, nullptr, (T*)nullptr, 0.f));
   else
-    SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 1>), dim3(rows, gy), dim3(NT), 0, st, X, mix, out_w, (const T*)y,
-                                 (const T*)parts, pw, K, S, W));
+    SM_T(f32, hipLaunchKernelGGL((hyper_update_kernel<T, 1, false>), dim3(rows, gy), dim3(NT), 0, st, X, mix, out_w,
+                                 (const T*)y, (const T*)parts, pw, K, S, W, nullptr, nullptr, (T*)nullptr, 0.f));
   return (int)hipGetLastError();
 }
 

@@ -763,14 +763,21 @@ def hyper_read_norm(X: torch.Tensor, in_w: Optional[torch.Tensor], weight: torch
 
 
 def hyper_update(X: torch.Tensor, mix: Optional[torch.Tensor], out_w: Optional[torch.Tensor], y: Optional[torch.Tensor],
-                 parts: Optional[torch.Tensor] = None, part_w: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 parts: Optional[torch.Tensor] = None, part_w: Optional[torch.Tensor] = None, nxt: Optional[tuple] = None):
     """X fp32 [T, S, W], in place, all streams at once from the old ones:
     X[:, r] <- sum_s mix[s, r] X[:, s] + out_w[r] v, with v = y + sum_k part_w[:, k] parts[:, k] summed in
     fp32 in k order (``y`` [T, W] or None; ``parts`` [T, K, W] with ``part_w`` fp32 [T, K]: a mixture's
-    expert outputs).  ``mix`` fp32 [S, S] indexed [from, to] and ``out_w`` fp32 [S]; both None: X += v."""
+    expert outputs).  ``mix`` fp32 [S, S] indexed [from, to] and ``out_w`` fp32 [S]; both None: X += v.
+    Returns X, or with ``nxt`` = (in_w, weight, eps) the next sublayer's input ``hyper_read_norm`` of the new
+    streams in the dtype of y / parts, computed in the same pass."""
     if _gpu(X):
-        _ext().sm_hyper_update(X, mix, out_w, y, parts, part_w)
+        if nxt is not None:
+            return _ext().sm_hyper_update(X, mix, out_w, y, parts, part_w, nxt[0], nxt[1], float(nxt[2]))
+        _ext().sm_hyper_update(X, mix, out_w, y, parts, part_w, None, None, 0.0)
         return X
+    if nxt is not None:
+        hyper_update(X, mix, out_w, y, parts, part_w)
+        return hyper_read_norm(X, nxt[0], nxt[1], nxt[2], (y if y is not None else parts).dtype)
     v = y.float() if y is not None else torch.zeros_like(X[:, 0])
     if parts is not None:
         for k in range(parts.shape[1]):

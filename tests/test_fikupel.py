@@ -228,6 +228,12 @@ def test_stream_read_norm_and_rebuild(dev, S, W):
         assert torch.allclose(got, want, atol=3e-5)
         got = seqmix.hyper_update(D(X.clone()), None, None, D(yy), D(pp), D(ww)).cpu().double()   # no stream weights: x + v
         assert torch.allclose(got, Xd + v[:, None, :], atol=3e-5)
+        for a2 in (a, None):                                  # the next sublayer's read + norm in the same pass
+            Xn = D(X.clone())
+            h = seqmix.hyper_update(Xn, D(M), D(b), D(yy), D(pp), D(ww), nxt=(D(a2), D(wn), 1e-5)).cpu().double()
+            assert torch.allclose(Xn.cpu().double(), want, atol=3e-5)
+            u = want.sum(1) if a2 is None else torch.einsum("s,tsw->tw", a2.double(), want)
+            assert torch.allclose(h, rms(u) * wn.double(), atol=3e-5)
 
 
 @pytest.mark.parametrize("dev", DEVS)
